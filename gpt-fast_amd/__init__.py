@@ -1,0 +1,17 @@
+"""An MI355X-native generation library for the Llama 2/3 dense decoder.
+
+From a model folder (``config.json`` + safetensors) or seeded random weights to
+generated tokens, through hand-written HIP kernels for gfx950:
+
+    from gpt_fast_amd import Engine, generate
+    engine = Engine.from_folder("path/to/model", dtype="bfloat16", max_tokens=8192)
+    out = generate(engine, [[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
+"""
+from . import architectures as _architectures          # registers the known architectures
+from .config.registry import (architecture, known_architectures, read_model_folder,
+                              register_architecture)
+from .engine.batch import Entry
+from .engine.step import Engine
+from .parts.base import (register_block, register_feed_forward, register_mixer, register_norm,
+                         register_position)
+from .weights.random_init import write_random_model

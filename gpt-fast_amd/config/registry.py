@@ -1,0 +1,77 @@
+"""The one registry from an architecture's name to its model.
+
+An :class:`Architecture` bundles what is particular to one model family: how its
+``config.json`` is read into a typed configuration, how that configuration becomes a
+:class:`~.spec.ModelPlan`, and how the tensors of its checkpoint files map to the
+plan's parameters.  Everything else in the library is shared.
+
+The reference picks its one model class by the checkpoint folder's name
+(generate.py:222, model.py:44-57, 148-150); here ``config.json`` names it through
+``architectures[0]`` or ``model_type``.
+"""
+import json
+import os
+from dataclasses import dataclass
+from typing import Callable, Dict, Tuple
+
+
+class UnknownArchitecture(KeyError):
+    pass
+
+
+@dataclass(frozen=True)
+class Architecture:
+    names: Tuple[str, ...]                      # e.g. ("LlamaForCausalLM", "llama")
+    read_config: Callable[[dict], object]       # config.json dict -> typed configuration
+    plan: Callable[[object], object]            # typed configuration -> ModelPlan
+    bindings: Callable[[object], list]          # typed configuration -> [weights.Binding]
+    config_dict: Callable[[object], dict]       # typed configuration -> config.json dict
+    presets: Callable[[str], object] = None     # preset name -> typed configuration
+
+
+_ARCHITECTURES: Dict[str, Architecture] = {}
+
+
+def register_architecture(arch: Architecture) -> Architecture:
+    for name in arch.names:
+        _ARCHITECTURES[name] = arch
+    return arch
+
+
+def known_architectures():
+    return sorted(_ARCHITECTURES)
+
+
+def architecture(name: str) -> Architecture:
+    try:
+        return _ARCHITECTURES[name]
+    except KeyError:
+        raise UnknownArchitecture(
+            f"unknown architecture '{name}'; known: {known_architectures()}") from None
+
+
+def architecture_of(config_json: dict) -> Architecture:
+    """The architecture that a ``config.json`` dictionary names."""
+    names = list(config_json.get("architectures") or [])
+    if config_json.get("model_type"):
+        names.append(config_json["model_type"])
+    if not names:
+        raise UnknownArchitecture(
+            "config.json has neither 'architectures' nor 'model_type'; "
+            f"known: {known_architectures()}")
+    for name in names:
+        if name in _ARCHITECTURES:
+            return _ARCHITECTURES[name]
+    raise UnknownArchitecture(
+        f"unknown architecture {names}; known: {known_architectures()}")
+
+
+def read_model_folder(folder: str):
+    """(architecture, typed configuration) of a model folder."""
+    path = os.path.join(folder, "config.json")
+    if not os.path.isfile(path):
+        raise FileNotFoundError(f"{path}: a model folder needs a config.json")
+    with open(path) as f:
+        raw = json.load(f)
+    arch = architecture_of(raw)
+    return arch, arch.read_config(raw)

@@ -1,0 +1,368 @@
+// Plain kernels for every op of a decoder step.
+//
+// These are the reference kernels of the library: simple, one workgroup per row or per
+// (token, head), all arithmetic in float.  The float32 engine runs on them alone; the
+// bfloat16 engine uses them where no faster kernel exists, and the faster kernels are
+// tested against them.  In each kernel the order of floating-point additions that
+// produce one output element depends only on that element's own inputs (its row, its
+// position), never on the number of rows or on the other sequences of the launch, so a
+// float32 result is the same however the tokens were cut into steps or batched.
+#include "common.h"
+
+// --------------------------------------------------------------------------------------
+// embedding gather: out[n, :] = float(table[tokens[n], :])          (model.py:140)
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ out, int dim) {
+    const int n = blockIdx.x;
+    const T* row = table + (size_t)tokens[n] * dim;
+    float* o = out + (size_t)n * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) o[d] = load_as_float(row + d);
+}
+
+extern "C" int gfa_embed(const void* table, int table_bf16, const int* tokens, float* out,
+                         int n_tokens, int dim, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (table_bf16)
+        embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)table, tokens, out, dim);
+    else
+        embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, tokens, out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// RMS norm: out[i, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w[:],  r = rows ? rows[i] : i
+// (model.py:236-241; statistics in float, one rounding at the store)
+template <typename T>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               const int* __restrict__ rows, T* __restrict__ out, int dim,
+                               float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    const float* xr = x + (size_t)r * dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        const float v = xr[d];
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float rs = rsqrtf(ss / (float)dim + eps);
+    T* o = out + (size_t)i * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) store_from_float(o + d, xr[d] * rs * w[d]);
+}
+
+extern "C" int gfa_rmsnorm(const float* x, const float* w, const int* rows, void* out,
+                           int out_bf16, int n_rows, int dim, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (out_bf16)
+        rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, w, rows, (bf16_t*)out, dim, eps);
+    else
+        rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>(x, w, rows, (float*)out, dim, eps);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// float32 matrix product: out[m, n] (+)= sum_k a[m, k] * w[n, k]
+// 64x64 tile per workgroup of 256 threads, 4x4 outputs per thread, k in steps of 16 through
+// shared memory.  Each output is one fused-multiply-add chain over k = 0..K-1 in order.
+#define GF_BM 64
+#define GF_BN 64
+#define GF_BK 16
+__global__ __launch_bounds__(256) void gemm_f32_kernel(
+        const float* __restrict__ a, const float* __restrict__ w, float* __restrict__ out,
+        int M, int N, int K, int lda, int ldo, int accumulate) {
+    __shared__ float As[GF_BK][GF_BM + 4];
+    __shared__ float Ws[GF_BK][GF_BN + 4];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = blockIdx.y * GF_BM, n0 = blockIdx.x * GF_BN;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += GF_BK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = threadIdx.x + i * 256;
+            const int r = e >> 4, c = e & 15;
+            const int k = k0 + c;
+            const int m = m0 + r, n = n0 + r;
+            As[c][r] = (m < M && k < K) ? a[(size_t)m * lda + k] : 0.f;
+            Ws[c][r] = (n < N && k < K) ? w[(size_t)n * K + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GF_BK; ++kk) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float* o = out + (size_t)m * ldo + n;
+            *o = accumulate ? (*o + acc[i][j]) : acc[i][j];
+        }
+    }
+}
+
+extern "C" int gfa_gemm_f32(const float* a, const float* w, float* out, int M, int N, int K,
+                            int lda, int ldo, int accumulate, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM);
+    gemm_f32_kernel<<<grid, 256, 0, stream>>>(a, w, out, M, N, K, lda, ldo, accumulate);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// Rotary position encoding of q and k, and the write of k and v into the paged cache.
+// qkv: [N, (H + 2*Hkv) * hd] rows of q heads, k heads, v heads (model.py:195-199).
+// Pair i of a head is (2i, 2i+1) if layout == 0 (model.py:281-293) or (i, i + rot/2) if
+// layout == 1; it is rotated by angle = float(position) * freqs[i], cos and sin in float.
+// Elements beyond `rot` pass through.  q goes to q_out [N, H, hd]; k and v of token n go
+// to page table[seq(n)][pos / PAGE], offset pos % PAGE (model.py:91-100, 206-207).
+template <typename T>
+__global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                                  T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                  const float* __restrict__ freqs,
+                                  const int* __restrict__ tok_seq,
+                                  const int* __restrict__ tok_pos,
+                                  const int* __restrict__ table, int table_stride, int H,
+                                  int Hkv, int hd, int rot, int layout) {
+    const int n = blockIdx.x;
+    const int pos = tok_pos[n];
+    const T* row = qkv + (size_t)n * (H + 2 * Hkv) * hd;
+    const int half = hd / 2;          // pairs per head when every element had a partner
+    const int rot_pairs = rot / 2;
+    size_t kv_base = 0;
+    if (k_pages) {
+        const int page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+        kv_base = page_row(page, 0, pos % GFA_PAGE, Hkv, hd);
+    }
+    // q and k heads: one thread per (head, pair-or-passthrough slot)
+    const int n_rot_heads = H + Hkv;
+    for (int e = threadIdx.x; e < n_rot_heads * half; e += blockDim.x) {
+        const int head = e / half, i = e % half;
+        const T* src = row + (size_t)head * hd;
+        T* dst;
+        if (head < H) {
+            dst = q_out + ((size_t)n * H + head) * hd;
+        } else {
+            if (!k_pages) continue;
+            dst = k_pages + kv_base + (size_t)(head - H) * GFA_PAGE * hd;
+        }
+        if (i < rot_pairs) {
+            const int ia = layout == 0 ? 2 * i : i;
+            const int ib = layout == 0 ? 2 * i + 1 : i + rot_pairs;
+            const float a = load_as_float(src + ia), b = load_as_float(src + ib);
+            float s, c;
+            sincosf((float)pos * freqs[i], &s, &c);
+            store_from_float(dst + ia, a * c - b * s);
+            store_from_float(dst + ib, b * c + a * s);
+        } else {
+            // elements rot .. hd-1 are copied, two per slot
+            const int d0 = rot + 2 * (i - rot_pairs);
+            dst[d0] = src[d0];
+            dst[d0 + 1] = src[d0 + 1];
+        }
+    }
+    if (v_pages) {
+        const T* vsrc = row + (size_t)(H + Hkv) * hd;
+        for (int e = threadIdx.x; e < Hkv * hd; e += blockDim.x) {
+            const int g = e / hd, d = e % hd;
+            v_pages[kv_base + (size_t)g * GFA_PAGE * hd + d] = vsrc[e];
+        }
+    }
+}
+
+extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages, void* v_pages,
+                                    const float* freqs, const int* tok_seq, const int* tok_pos,
+                                    const int* table, int table_stride, int n_tokens, int H,
+                                    int Hkv, int hd, int rot, int layout, int is_bf16,
+                                    hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (is_bf16)
+        rope_cache_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(
+            (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs,
+            tok_seq, tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
+    else
+        rope_cache_kernel<float><<<n_tokens, 256, 0, stream>>>(
+            (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, freqs, tok_seq,
+            tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// Attention of each new token over its sequence's cache (model.py:209-211 with the mask of
+// model.py:134,138): query head h reads kv head h / (H/Hkv); keys j with
+// max(0, pos-window+1) <= j <= pos (window 0: from 0); scores scaled, softmax with running
+// maximum, all in float.  One workgroup of 128 threads per (head, token); keys in chunks of
+// 128, one key per thread for the scores, one output element per thread for the values.
+#define AG_THREADS 128
+#define AG_MAX_PER_THREAD 4            // head_dim <= 512
+template <typename T>
+__global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
+        const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, int table_stride, T* __restrict__ out, int H, int Hkv,
+        int hd, float scale, int window) {
+    extern __shared__ float shared[];
+    float* qs = shared;                 // [hd]
+    float* sc = shared + hd;            // [AG_THREADS]
+    float* scratch = sc + AG_THREADS;   // [16]
+    const int h = blockIdx.x, n = blockIdx.y;
+    const int g = h / (H / Hkv);
+    const int pos = tok_pos[n];
+    const int* pages = table + (size_t)tok_seq[n] * table_stride;
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const T* qrow = q + ((size_t)n * H + h) * hd;
+    for (int d = threadIdx.x; d < hd; d += AG_THREADS) qs[d] = load_as_float(qrow + d);
+    __syncthreads();
+
+    float m = -INFINITY, l = 0.f;
+    float acc[AG_MAX_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < AG_MAX_PER_THREAD; ++i) acc[i] = 0.f;
+
+    for (int base = lo; base <= pos; base += AG_THREADS) {
+        const int j = base + threadIdx.x;
+        float s = -INFINITY;
+        if (j <= pos) {
+            const T* kr = k_pages + page_row(pages[j / GFA_PAGE], g, j % GFA_PAGE, Hkv, hd);
+            float dot = 0.f;
+            for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], load_as_float(kr + d), dot);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m, block_max(s, scratch));
+        const float alpha = expf(m - m_new);          // 0 on the first chunk (m = -inf)
+        const float p = (j <= pos) ? expf(s - m_new) : 0.f;
+        sc[threadIdx.x] = p;
+        l = l * alpha + block_sum(p, scratch);        // contains the barrier that publishes sc
+        const int count = (pos - base + 1 < AG_THREADS) ? pos - base + 1 : AG_THREADS;
+#pragma unroll
+        for (int i = 0; i < AG_MAX_PER_THREAD; ++i) {
+            const int d = threadIdx.x + i * AG_THREADS;
+            if (d < hd) {
+                float a = acc[i] * alpha;
+                for (int jj = 0; jj < count; ++jj) {
+                    const int key = base + jj;
+                    const T* vr = v_pages + page_row(pages[key / GFA_PAGE], g, key % GFA_PAGE,
+                                                     Hkv, hd);
+                    a = fmaf(sc[jj], load_as_float(vr + d), a);
+                }
+                acc[i] = a;
+            }
+        }
+        m = m_new;
+        __syncthreads();
+    }
+    T* orow = out + ((size_t)n * H + h) * hd;
+#pragma unroll
+    for (int i = 0; i < AG_MAX_PER_THREAD; ++i) {
+        const int d = threadIdx.x + i * AG_THREADS;
+        if (d < hd) store_from_float(orow + d, acc[i] / l);
+    }
+}
+
+extern "C" int gfa_attention_generic(const void* q, const void* k_pages, const void* v_pages,
+                                     const int* tok_seq, const int* tok_pos, const int* table,
+                                     int table_stride, void* out, int n_tokens, int H, int Hkv,
+                                     int hd, float scale, int window, int is_bf16,
+                                     hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (hd > AG_THREADS * AG_MAX_PER_THREAD) return (int)hipErrorInvalidValue;
+    dim3 grid(H, n_tokens);
+    const size_t shmem = (size_t)(hd + AG_THREADS + 16) * sizeof(float);
+    if (is_bf16)
+        attention_generic_kernel<bf16_t><<<grid, AG_THREADS, shmem, stream>>>(
+            (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, tok_seq, tok_pos,
+            table, table_stride, (bf16_t*)out, H, Hkv, hd, scale, window);
+    else
+        attention_generic_kernel<float><<<grid, AG_THREADS, shmem, stream>>>(
+            (const float*)q, (const float*)k_pages, (const float*)v_pages, tok_seq, tok_pos,
+            table, table_stride, (float*)out, H, Hkv, hd, scale, window);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// gate: out[n, i] = act(gu[n, i]) * gu[n, I + i], act = silu (model.py:227)
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I,
+                                size_t total) {
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
+         e += (size_t)gridDim.x * blockDim.x) {
+        const size_t n = e / I;
+        const int i = (int)(e % I);
+        const float a = load_as_float(gu + n * 2 * I + i);
+        const float b = load_as_float(gu + n * 2 * I + I + i);
+        store_from_float(out + e, (a / (1.f + expf(-a))) * b);
+    }
+}
+
+extern "C" int gfa_silu_mul(const void* gu, void* out, int n_rows, int I, int is_bf16,
+                            hipStream_t stream) {
+    const size_t total = (size_t)n_rows * I;
+    if (total == 0) return 0;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (is_bf16)
+        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+    else
+        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// residual sum in float: res[e] += float(y[e])          (model.py:162-163)
+template <typename T>
+__global__ void add_into_kernel(float* __restrict__ res, const T* __restrict__ y, size_t total) {
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
+         e += (size_t)gridDim.x * blockDim.x)
+        res[e] += load_as_float(y + e);
+}
+
+extern "C" int gfa_add_into(float* res, const void* y, size_t total, int y_bf16,
+                            hipStream_t stream) {
+    if (total == 0) return 0;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (y_bf16)
+        add_into_kernel<bf16_t><<<blocks, 256, 0, stream>>>(res, (const bf16_t*)y, total);
+    else
+        add_into_kernel<float><<<blocks, 256, 0, stream>>>(res, (const float*)y, total);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// naive matrix product with bfloat16 operands and float accumulation, one thread per
+// output: the plain counterpart of the fast bfloat16 kernels (tests only).
+__global__ void gemm_bf16_naive_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                       float* __restrict__ out, int M, int N, int K) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x, m = blockIdx.y;
+    if (n >= N || m >= M) return;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k)
+        acc = fmaf(bf16_to_float(a[(size_t)m * K + k]), bf16_to_float(w[(size_t)n * K + k]), acc);
+    out[(size_t)m * N + n] = acc;
+}
+
+extern "C" int gfa_gemm_bf16_naive(const void* a, const void* w, float* out, int M, int N, int K,
+                                   hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    dim3 grid((N + 255) / 256, M);
+    gemm_bf16_naive_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, out, M, N, K);
+    return GFA_LAUNCH_RESULT();
+}

@@ -1,0 +1,59 @@
+"""Matrix products of the step, ``y = x W^T`` with ``W`` stored ``[out, in]`` as in the
+reference's linears (model.py:110, 174-175, 222-224), with the epilogues the blocks need.
+
+float32 engine: the library's own float32 kernel, for every shape (a true 32-bit
+product; one fused-multiply-add chain per output).
+
+bfloat16 engine: hand-written kernels for the few-row products of decoding (weights are
+streamed once; see csrc/gemm_bf16.hip); the vendor matrix library, through
+``torch.matmul``, for the many-row products of prefill - the reference uses the vendor
+library for these as well.  Accumulation is float32 everywhere.
+"""
+from typing import Optional
+
+import torch
+
+from . import kernels as K
+from .library import KernelError
+
+# products with at most this many rows go to the hand-written streaming kernels
+SKINNY_MAX_ROWS = 64
+
+
+def _fast():
+    from . import gemm_bf16
+    return gemm_bf16
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+    """[M, N] = x [M, K] times w [N, K] transposed, in ``out_dtype`` (default: x's)."""
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise KernelError("a float32 product has a float32 result")
+        return K.gemm_f32(x, w)
+    M = x.shape[0]
+    if M <= SKINNY_MAX_ROWS:
+        return _fast().skinny(x, w, out_dtype=out_dtype)
+    if out_dtype == torch.float32:
+        return _fast().wide_f32_out(x, w)
+    return torch.matmul(x, w.t())
+
+
+def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor):
+    """residual (float32 [M, N]) += x W^T."""
+    if x.dtype == torch.float32:
+        return K.gemm_f32(x, w, out=residual, accumulate=True)
+    if x.shape[0] <= SKINNY_MAX_ROWS:
+        return _fast().skinny(x, w, residual=residual)
+    return K.add_into(residual, torch.matmul(x, w.t()))
+
+
+def gated_linear(x: torch.Tensor, w13: torch.Tensor):
+    """[M, I] = silu(x W1^T) * (x W3^T), with w13 = rows of W1 then rows of W3
+    (model.py:227)."""
+    if x.dtype == torch.float32:
+        return K.silu_mul(K.gemm_f32(x, w13))
+    if x.shape[0] <= SKINNY_MAX_ROWS:
+        return _fast().skinny_gated(x, w13)
+    return K.silu_mul(torch.matmul(x, w13.t()))

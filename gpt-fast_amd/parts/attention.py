@@ -1,0 +1,52 @@
+"""Causal attention with grouped key/value heads over the paged cache
+(reference model.py:167-216)."""
+import torch
+
+from ..cache.store import KVNeed
+from ..config.spec import AttentionSpec
+from ..ops import attention as A
+from ..ops import kernels as K
+from ..ops import linear as L
+from .base import POSITIONS, Param, Part, Runtime, check_bound, register_mixer
+
+
+class Attention(Part):
+    """``wo( softmax(q k^T * scale + causal mask) v )`` with q, k, v = split(wqkv x),
+    positions applied to q and k by the spec's position encoding, k and v written to the
+    cache entry before they are read.  Query head h reads kv head h // (H / Hkv)
+    (model.py:209-210).  Scores, softmax and the weighted sum are float32."""
+
+    def __init__(self, spec: AttentionSpec, runtime: Runtime):
+        if spec.n_heads % spec.n_kv_heads:
+            raise ValueError(f"{spec.n_heads} heads do not divide into {spec.n_kv_heads} kv heads")
+        self.spec = spec
+        self.rt = runtime
+        self.position = POSITIONS.build(spec.position, runtime)
+        self.scale = spec.scale if spec.scale is not None else K.default_scale(spec.head_dim)
+        self.window = 0 if spec.window is None else int(spec.window)
+        self.wqkv = self.wo = None
+
+    def parameters(self):
+        s = self.spec
+        return {"wqkv": Param(((s.n_heads + 2 * s.n_kv_heads) * s.head_dim, s.dim)),
+                "wo": Param((s.dim, s.n_heads * s.head_dim))}
+
+    def bind(self, tensors):
+        check_bound("Attention", self.parameters(), tensors)
+        self.wqkv, self.wo = tensors["wqkv"], tensors["wo"]
+
+    def cache_need(self):
+        s = self.spec
+        return KVNeed(s.n_kv_heads, s.head_dim, s.window)
+
+    def forward(self, x, batch, entry, residual):
+        s = self.spec
+        qkv = L.linear(x, self.wqkv)                                        # model.py:195
+        q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
+                                           s.head_dim)                      # model.py:201-207
+        y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
+                        self.scale, self.window)                            # model.py:209-211
+        L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual)  # :215, 162
+
+
+register_mixer("attention", Attention)

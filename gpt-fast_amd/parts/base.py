@@ -1,0 +1,112 @@
+"""Interfaces of the parts a layer is made of, and the registries that map a spec's
+``kind`` to the part that runs it.
+
+A part is built from its spec and a :class:`Runtime`, states the parameters it owns
+(:meth:`Part.parameters`), receives them (:meth:`Part.bind`) and then runs.  No part knows
+which model it is in; it sees its own spec, the step's batch and its own cache entry.
+
+Interfaces (N = tokens of the step, D = model width):
+
+* norm:          ``forward(residual float32 [N, D], rows=None) -> [n, D]`` in the compute type
+* mixer:         ``cache_need() -> KVNeed | StateNeed | None``;
+                 ``forward(x [N, D], batch, entry, residual)`` adds its output into
+                 ``residual`` (float32 [N, D], in place)
+* feed-forward:  ``forward(x [N, D], batch, residual)`` adds its output into ``residual``
+* position:      ``rotate_and_store(qkv, batch, entry, n_heads, n_kv_heads, head_dim) -> q``
+* block:         ``forward(residual, batch, entry)`` updates ``residual`` in place
+
+A new part is a class with these methods, registered under a new ``kind``; its spec is
+any object with that ``kind`` attribute.
+"""
+from dataclasses import dataclass
+from typing import Callable, Dict, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class Param:
+    """A parameter a part owns: shape, role ("matrix" | "vector" | "index", as in
+    weights.bindings) and how random weights draw it."""
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "linear"
+
+
+class Runtime:
+    """What parts need to know about the engine they run in."""
+
+    def __init__(self, dtype: torch.dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"compute type {dtype}: float32 or bfloat16")
+        self.dtype = dtype
+        self.device = torch.device(device)
+
+    @property
+    def is_float32(self) -> bool:
+        return self.dtype == torch.float32
+
+
+class Part:
+    def parameters(self) -> Dict[str, Param]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        pass
+
+
+class _Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._kinds: Dict[str, Callable] = {}
+
+    def register(self, kind: str, factory: Callable) -> Callable:
+        self._kinds[kind] = factory
+        return factory
+
+    def build(self, spec, runtime: Runtime):
+        kind = getattr(spec, "kind", None)
+        if kind not in self._kinds:
+            raise KeyError(f"no {self.what} is registered for kind '{kind}'; "
+                           f"known: {sorted(self._kinds)}")
+        return self._kinds[kind](spec, runtime)
+
+    def kinds(self):
+        return sorted(self._kinds)
+
+
+NORMS = _Registry("norm")
+POSITIONS = _Registry("position encoding")
+MIXERS = _Registry("mixer")
+FEED_FORWARDS = _Registry("feed-forward")
+BLOCKS = _Registry("block arrangement")      # keyed by LayerSpec.arrangement
+
+
+def register_norm(kind, factory):
+    return NORMS.register(kind, factory)
+
+
+def register_position(kind, factory):
+    return POSITIONS.register(kind, factory)
+
+
+def register_mixer(kind, factory):
+    return MIXERS.register(kind, factory)
+
+
+def register_feed_forward(kind, factory):
+    return FEED_FORWARDS.register(kind, factory)
+
+
+def register_block(arrangement, factory):
+    return BLOCKS.register(arrangement, factory)
+
+
+def check_bound(owner: str, declared: Dict[str, Param], tensors: Dict[str, torch.Tensor]) -> None:
+    """Every declared parameter is there with its shape."""
+    for name, p in declared.items():
+        if name not in tensors:
+            raise KeyError(f"{owner}: parameter '{name}' was not given")
+        if tuple(tensors[name].shape) != tuple(p.shape):
+            raise ValueError(f"{owner}: parameter '{name}' is {list(tensors[name].shape)}, "
+                             f"expected {list(p.shape)}")

@@ -1,0 +1,44 @@
+"""How norms, mixer, feed-forward and the residual stream are wired in one layer."""
+from ..config.spec import LayerSpec
+from .base import FEED_FORWARDS, MIXERS, NORMS, Part, Runtime, register_block
+
+
+class PreNormBlock(Part):
+    """``h = x + mixer(norm1(x)); out = h + ffn(norm2(h))`` (reference model.py:161-164).
+    The residual stream is float32 and updated in place; the sums happen in the
+    parts' epilogues."""
+
+    def __init__(self, spec: LayerSpec, runtime: Runtime):
+        self.spec = spec
+        self.mixer_norm = NORMS.build(spec.mixer_norm, runtime)
+        self.mixer = MIXERS.build(spec.mixer, runtime)
+        self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, runtime)
+        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, runtime)
+
+    def children(self):
+        s = self.spec
+        return {s.mixer_norm_name: self.mixer_norm, s.mixer_name: self.mixer,
+                s.feed_forward_norm_name: self.feed_forward_norm,
+                s.feed_forward_name: self.feed_forward}
+
+    def parameters(self):
+        out = {}
+        for child_name, child in self.children().items():
+            for name, p in child.parameters().items():
+                out[f"{child_name}.{name}"] = p
+        return out
+
+    def bind(self, tensors):
+        for child_name, child in self.children().items():
+            prefix = child_name + "."
+            child.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, residual, batch, entry):
+        self.mixer.forward(self.mixer_norm.forward(residual), batch, entry, residual)
+        self.feed_forward.forward(self.feed_forward_norm.forward(residual), batch, residual)
+
+
+register_block("pre_norm", PreNormBlock)

@@ -1,0 +1,31 @@
+"""Gated feed-forward (reference model.py:219-227)."""
+from ..config.spec import GatedFeedForwardSpec
+from ..ops import linear as L
+from .base import Param, Part, Runtime, check_bound, register_feed_forward
+
+
+class GatedFeedForward(Part):
+    """``w2( silu(w1 x) * (w3 x) )`` without biases.  w1 and w3 are one matrix ``w13``
+    (rows of w1, then rows of w3) so that the gate is applied where the products end."""
+
+    def __init__(self, spec: GatedFeedForwardSpec, runtime: Runtime):
+        if spec.activation != "silu":
+            raise ValueError(f"activation '{spec.activation}': only silu has a kernel")
+        self.spec = spec
+        self.rt = runtime
+        self.w13 = self.w2 = None
+
+    def parameters(self):
+        s = self.spec
+        return {"w13": Param((2 * s.hidden, s.dim)), "w2": Param((s.dim, s.hidden))}
+
+    def bind(self, tensors):
+        check_bound("GatedFeedForward", self.parameters(), tensors)
+        self.w13, self.w2 = tensors["w13"], tensors["w2"]
+
+    def forward(self, x, batch, residual):
+        h = L.gated_linear(x, self.w13)
+        L.linear_into(h, self.w2, residual)
+
+
+register_feed_forward("gated", GatedFeedForward)

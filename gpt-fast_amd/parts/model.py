@@ -1,0 +1,93 @@
+"""A whole decoder assembled from a plan (reference model.py:102-146)."""
+from typing import Dict, List
+
+import torch
+
+from ..config.spec import ModelPlan
+from ..ops import kernels as K
+from ..ops import linear as L
+from .base import BLOCKS, NORMS, Param, Runtime, check_bound
+
+
+class DecoderModel:
+    """Embedding, the plan's layers in the plan's order, final norm, output head.
+
+    ``forward`` runs the tokens of one step: embeds them, passes the float32 residual
+    stream through every run of the order with that run's cache entry, then norms and
+    projects only the rows whose logits are wanted (the reference projects every
+    position, model.py:144-146)."""
+
+    def __init__(self, plan: ModelPlan, runtime: Runtime):
+        plan.validate()
+        self.plan = plan
+        self.rt = runtime
+        self.blocks = [BLOCKS.build(_Arranged(layer), runtime) for layer in plan.layers]
+        self.final_norm = NORMS.build(plan.final_norm, runtime)
+        self.embedding = self.head = None
+
+    # ------------------------------------------------------------------ parameters
+    def parameters(self) -> Dict[str, Param]:
+        p = {self.plan.embedding_name: Param((self.plan.vocab_size, self.plan.dim)),
+             self.plan.head_name: Param((self.plan.vocab_size, self.plan.dim)),
+             self.plan.final_norm_name: Param((self.plan.dim,), "vector", "norm")}
+        for layer, block in zip(self.plan.layers, self.blocks):
+            for name, param in block.parameters().items():
+                p[f"{layer.name}.{name}"] = param
+        return p
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        declared = self.parameters()
+        check_bound("model", declared, tensors)
+        extra = sorted(set(tensors) - set(declared))
+        if extra:
+            raise KeyError(f"model: parameters {extra} belong to no part")
+        self._tensors = dict(tensors)
+        self.embedding = tensors[self.plan.embedding_name]
+        self.head = tensors[self.plan.head_name]
+        self.final_norm.bind({"weight": tensors[self.plan.final_norm_name]})
+        for layer, block in zip(self.plan.layers, self.blocks):
+            prefix = layer.name + "."
+            block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+
+    def parameter_bytes(self, exclude_embedding: bool = True) -> int:
+        """Bytes of the parameters one decode step reads (the embedding table is a
+        gather of a few rows, as in the reference's accounting, generate.py:251-268)."""
+        seen, total = set(), 0
+        for name, t in self._tensors.items():
+            if exclude_embedding and name == self.plan.embedding_name \
+                    and t.data_ptr() != self.head.data_ptr():
+                continue
+            if t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+        return total
+
+    # ------------------------------------------------------------------ cache
+    def cache_needs(self) -> List[object]:
+        return [self.blocks[run.layer].cache_need() for run in self.plan.order]
+
+    def cache_borrow(self) -> List[object]:
+        return [run.cache_from for run in self.plan.order]
+
+    # ------------------------------------------------------------------ step
+    def forward(self, batch, cache) -> torch.Tensor:
+        """float32 logits [n_wanted, vocab] of the step described by ``batch``."""
+        residual = K.embed(self.embedding, batch.tokens)                  # model.py:140
+        for n, run in enumerate(self.plan.order):                         # model.py:142-143
+            self.blocks[run.layer].forward(residual, batch, cache.entries[n])
+        if batch.n_want == 0:
+            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32,
+                               device=residual.device)
+        x = self.final_norm.forward(residual, rows=batch.want_rows)       # model.py:144
+        return L.linear(x, self.head, out_dtype=torch.float32)            # model.py:145
+
+
+class _Arranged:
+    """Gives a LayerSpec the ``kind`` its arrangement is registered under."""
+
+    def __init__(self, layer):
+        self._layer = layer
+        self.kind = layer.arrangement
+
+    def __getattr__(self, name):
+        return getattr(self._layer, name)

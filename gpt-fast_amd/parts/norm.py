@@ -1,0 +1,30 @@
+"""RMS norm (reference model.py:230-241)."""
+import torch
+
+from ..config.spec import NormSpec
+from ..ops import kernels as K
+from .base import Param, Part, Runtime, check_bound, register_norm
+
+
+class RMSNorm(Part):
+    """``x * rsqrt(mean(x^2) + eps) * weight`` over the last dimension; statistics and
+    scaling in float32 from the float32 residual stream, one rounding to the compute type
+    at the store.  ``eps`` and the width are the spec's."""
+
+    def __init__(self, spec: NormSpec, runtime: Runtime):
+        self.spec = spec
+        self.rt = runtime
+        self.weight = None
+
+    def parameters(self):
+        return {"weight": Param((self.spec.dim,), role="vector", init="norm")}
+
+    def bind(self, tensors):
+        check_bound("RMSNorm", self.parameters(), tensors)
+        self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+    def forward(self, residual: torch.Tensor, rows=None) -> torch.Tensor:
+        return K.rmsnorm(residual, self.weight, self.spec.eps, self.rt.dtype, rows=rows)
+
+
+register_norm("rms", RMSNorm)

@@ -1,0 +1,99 @@
+"""The engine against the plain implementation on the GPU: whole prompts, token by
+token, unequal batches with slot reuse, float32 and bfloat16."""
+import pytest
+import torch
+
+import util
+from util import TOL_BF16, TOL_F32, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [("float32", TOL_F32), ("bfloat16", TOL_BF16)]
+
+
+def engine_for(folder, dtype, max_tokens=4096):
+    import gpt_fast_amd as gfa
+    return gfa.Engine.from_folder(folder, dtype=dtype, device="cuda:0", max_tokens=max_tokens)
+
+
+def whole(engine, tokens):
+    from gpt_fast_amd import Entry
+    slot = engine.start_sequence()
+    logits = engine.step([Entry(slot, tokens, want=list(range(len(tokens))))])
+    engine.end_sequence(slot)
+    return logits.cpu()
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_whole_prompt(tmp_path_factory, name, dtype, tol):
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype)
+    V = util.TINY[name]["vocab_size"]
+    for n, seed in ((1, 1), (7, 2), (64, 3), (65, 4), (150, 5)):
+        tokens = util.random_tokens(V, n, seed)
+        want = util.plain_logits(folder, tokens)
+        got = whole(eng, tokens)
+        assert got.shape == want.shape
+        assert rel_err(got, want) < tol, (name, dtype, n)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_last_32_one_by_one(tmp_path_factory, name, dtype, tol):
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype)
+    V = util.TINY[name]["vocab_size"]
+    tokens = util.random_tokens(V, 100, 11)
+    want = util.plain_logits(folder, tokens)
+    slot = eng.start_sequence()
+    head = tokens[:-32]
+    got = [eng.step([Entry(slot, head, want=list(range(len(head))))]).cpu()]
+    for t in tokens[-32:]:
+        got.append(eng.step([Entry(slot, [t], want=[0])]).cpu())
+    eng.end_sequence(slot)
+    got = torch.cat(got)
+    assert rel_err(got, want) < tol
+    if dtype == "float32":
+        # a float32 result does not depend on the cutting at all
+        assert torch.equal(got, whole(eng, tokens))
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_unequal_batches_reuse_slots(tmp_path_factory, name, dtype, tol):
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype, max_tokens=64 * 12)
+    V = util.TINY[name]["vocab_size"]
+    for round_, lengths in enumerate(([7, 3, 12], [1, 5, 17, 33], [70, 2, 130, 64], [40, 90])):
+        new = [9, 4, 14, 6][:len(lengths)]
+        seqs = [util.random_tokens(V, L + n, 100 * round_ + i)
+                for i, (L, n) in enumerate(zip(lengths, new))]
+        slots = [eng.start_sequence() for _ in seqs]
+        got = [[] for _ in seqs]
+        # all prompts in one step
+        logits = eng.step([Entry(s, q[:L], want=list(range(L)))
+                           for s, q, L in zip(slots, seqs, lengths)]).cpu()
+        at = 0
+        for i, L in enumerate(lengths):
+            got[i].append(logits[at:at + L])
+            at += L
+        # then one token each; shorter requests end earlier
+        live = list(range(len(seqs)))
+        t = 0
+        while live:
+            logits = eng.step([Entry(slots[i], [seqs[i][lengths[i] + t]], want=[0])
+                               for i in live]).cpu()
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1])
+            t += 1
+            for i in [i for i in live if t >= new[i]]:
+                eng.end_sequence(slots[i])
+                live.remove(i)
+        for i, q in enumerate(seqs):
+            want = util.plain_logits(folder, q)
+            assert rel_err(torch.cat(got[i]), want) < tol, (name, dtype, round_, i)
+        eng.cache.check()
+    assert eng.cache.slots.held == 0

@@ -1,0 +1,71 @@
+"""Helpers shared by the tests: the tiny configurations, model folders made in a
+temporary directory, and the comparison of engine logits with the plain implementation."""
+import os
+import random
+
+import torch
+
+import plain_llama as plain
+
+# Two tiny configurations that differ in every size and option: heads and groups, head
+# size, widths that are no power of two, layers, vocabulary, eps, rope base and scaling.
+TINY_A = {   # Llama-2 style, MHA, no scaling
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 4,
+    "num_key_value_heads": 4, "intermediate_size": 176, "vocab_size": 256,
+    "max_position_embeddings": 64, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
+    "rope_scaling": None, "tie_word_embeddings": False,
+}
+TINY_B = {   # Llama-3.1 style, GQA 6:2, llama3 scaling whose three branches all occur
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 192, "num_hidden_layers": 3, "num_attention_heads": 6,
+    "num_key_value_heads": 2, "intermediate_size": 512, "vocab_size": 384,
+    "max_position_embeddings": 128, "rope_theta": 500000.0, "rms_norm_eps": 1e-6,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 32},
+    "tie_word_embeddings": False,
+}
+TINY_C = {   # odd sizes: head_dim given and != hidden/heads, GQA 5:1... width 200, vocab 1000
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 200, "num_hidden_layers": 2, "num_attention_heads": 10,
+    "num_key_value_heads": 5, "head_dim": 48, "intermediate_size": 328, "vocab_size": 1000,
+    "max_position_embeddings": 512, "rope_theta": 50000.0, "rms_norm_eps": 3e-6,
+    "rope_scaling": None, "tie_word_embeddings": True,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def make_folder(tmp, name, seed=0, dtype="float32", std=0.05):
+    """A model folder with random weights, written by the library's random-weights mode.
+    std 0.05 rather than 0.02 so that logits of these tiny models are not all near zero."""
+    import gpt_fast_amd as gfa
+    arch = gfa.config.registry.architecture_of(TINY[name])
+    cfg = arch.read_config(TINY[name])
+    folder = os.path.join(str(tmp), f"tiny_{name}_{dtype}_{seed}")
+    if not os.path.isdir(folder):
+        gfa.write_random_model(folder, arch, cfg, seed=seed, dtype=dtype, std=std)
+    return folder
+
+
+def random_tokens(vocab, n, seed):
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+def plain_logits(folder, tokens, dtype=torch.float32):
+    cfg, w = plain.load_folder(folder, dtype)
+    return plain.forward(w, cfg, tokens)
+
+
+def rel_err(a, b):
+    """Largest difference relative to the largest magnitude of the reference."""
+    a = a.double().cpu()
+    b = b.double().cpu()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+# Tolerances, stated once.  float32: the engine and the plain implementation do the same
+# arithmetic in different orders.  bfloat16: weights are bfloat16 in both; the engine
+# also rounds activations to bfloat16 between kernels.
+TOL_F32 = 2e-5
+TOL_BF16 = 4e-2

@@ -1,0 +1,169 @@
+"""Decode and prefill throughput of the Llama-3.1-8B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of a batch of 8 sequences (128-token random prompts, cache of
+4,096 positions per sequence, random bfloat16 weights, greedy sampling on the device).
+W untimed steps, then exactly K timed steps between device synchronisations.  Prints one
+JSON line: ``value`` is decoded tokens per second; ``prefill`` is one 2,048-token prompt;
+``roofline`` compares the bytes a decode step must read (every weight once, the cache of
+the live sequences) per second with the HBM peak; ``points`` holds decode at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                 # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+BASELINE_TOK_S = 93.89                # reference README: Llama-3.1-8B bf16, batch 1, A100
+
+
+def log(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def decode_run(engine, batch, prompt_len, warmup, steps, use_graph=True):
+    """(seconds per step, bytes a step reads) for `steps` decode steps of `batch` sequences."""
+    import torch
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.engine.decode import DecodeSession
+    from gpt_fast_amd.sampling import SamplingParams, sample
+    g = torch.Generator().manual_seed(batch)
+    V = engine.vocab_size
+    slots = [engine.start_sequence() for _ in range(batch)]
+    entries = [Entry(s, torch.randint(0, V, (prompt_len,), generator=g).tolist(),
+                     want=[prompt_len - 1], key=i) for i, s in enumerate(slots)]
+    params = SamplingParams(temperature=0.0)
+    # prefill in pieces of at most 8 prompts to bound activation memory
+    first = []
+    for i in range(0, batch, 8):
+        b = engine.prepare(entries[i:i + 8])
+        logits = engine.model.forward(b, engine.cache)
+        first.append(sample(logits, params, b.row_keys, None))
+    first = torch.cat(first)
+    sess = DecodeSession(engine, slots, list(range(batch)), first, params, use_graph=use_graph,
+                         max_new_tokens=warmup + steps + 1)
+    for _ in range(warmup):
+        sess.advance()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sess.advance()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    # bytes of the middle step: weights once + keys and values of every live token
+    ctx = prompt_len + warmup + steps // 2
+    kv_bytes = sum(g.bytes_per_token() for _, g in engine.cache.kv_groups) * ctx * batch
+    step_bytes = engine.model.parameter_bytes() + kv_bytes
+    for s in slots:
+        engine.end_sequence(s)
+    return dt, step_bytes
+
+
+def prefill_run(engine, n_tokens, repeats=3):
+    import torch
+    from gpt_fast_amd import Entry
+    g = torch.Generator().manual_seed(7)
+    toks = torch.randint(0, engine.vocab_size, (n_tokens,), generator=g).tolist()
+    best = None
+    for r in range(repeats + 1):
+        slot = engine.start_sequence()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([Entry(slot, toks, want=[n_tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.end_sequence(slot)
+        if r > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def prefill_flops(cfg, n_layers, T):
+    D, H, G, hd, I, V = (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads,
+                         cfg.head_dim, cfg.intermediate_size, cfg.vocab_size)
+    per_layer = (H + 2 * G) * hd * D + H * hd * D + 3 * I * D
+    linear = 2.0 * T * n_layers * per_layer
+    attn = n_layers * 2.0 * 2.0 * H * hd * (T * (T + 1) / 2)      # causal QK^T and PV
+    head = 2.0 * D * V                                             # last row only
+    return linear + attn + head
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this library")
+        sys.exit(2)
+
+    import torch
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.config.llama import LlamaConfig, preset_dict
+
+    raw = preset_dict("llama-3.1-8b")
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = LlamaConfig.from_dict(raw)
+    batch, context, prompt_len = 8, 4096, 128
+    t0 = time.time()
+    engine = gfa.Engine.from_random("llama", cfg, seed=0, dtype="bfloat16", device="cuda:0",
+                                    max_tokens=64 * context, max_sequences=64)
+    torch.cuda.synchronize()
+    log(f"[bench] model ready in {time.time() - t0:.1f} s")
+
+    use_graph = not args.no_graph
+    dt, step_bytes = decode_run(engine, batch, prompt_len, args.warmup, args.steps, use_graph)
+    value = batch / dt
+    log(f"[bench] decode b{batch}: {dt * 1e3:.3f} ms/step, {value:.1f} tok/s")
+    out = {
+        "metric": "decode tok/s @ batch 8; Llama-3.1-8B bf16", "value": round(value, 2),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / BASELINE_TOK_S, 3), "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "model": "llama-3.1-8b", "n_layer": cfg.num_hidden_layers,
+            "n_layer_full": full_layers, "dim": cfg.hidden_size,
+            "n_head": cfg.num_attention_heads, "n_kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size,
+            "vocab_size": cfg.vocab_size, "rope_base": cfg.rope_theta,
+            "rope_scaling": "llama3 factor 8 low 1 high 4 orig 8192",
+            "norm_eps": cfg.rms_norm_eps, "global_batch": batch, "seq_len": context,
+            "prompt_len": prompt_len, "new_tokens": args.warmup + args.steps,
+            "weights": "random N(0,0.02) bf16", "sampling": "greedy", "hip_graph": use_graph,
+            "parallelism": "single GPU",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(step_bytes / dt / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        T = 2048
+        pt = prefill_run(engine, T)
+        flops = prefill_flops(cfg, cfg.num_hidden_layers, T)
+        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                          "frac": round(flops / pt / 1e12 / MFMA_PEAK_TFLOPS["bf16"], 4)}
+        log(f"[bench] prefill {T}: {pt * 1e3:.2f} ms")
+        points = {}
+        for b in (1, 64):
+            steps = min(args.steps, 128)
+            d, _ = decode_run(engine, b, prompt_len, min(args.warmup, 8), steps, use_graph)
+            points[f"decode_b{b}"] = round(b / d, 2)
+            log(f"[bench] decode b{b}: {d * 1e3:.3f} ms/step, {b / d:.1f} tok/s")
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -15,3 +15,7 @@ from .engine.step import Engine
 from .parts.base import (register_block, register_feed_forward, register_mixer, register_norm,
                          register_position)
 from .weights.random_init import write_random_model
+from .engine.generate import GenerationResult, generate
+from .engine.cli import main
+from .sampling import SamplingParams
+from . import config, weights, parts, cache, engine, sampling, ops

@@ -1,0 +1,172 @@
+"""Command line in the manner of the reference's generate.py (its flags at
+generate.py:450-463, its driver at :272-437).
+
+    python -m gpt_fast_amd --checkpoint_path MODEL_FOLDER --prompt "Hello, my name is"
+    python -m gpt_fast_amd --random llama-3.1-8b --prompt 128 --batch_size 8
+
+``--checkpoint_path`` names a model *folder* (config.json + safetensors; the reference
+takes a converted model.pth whose folder name selects the configuration,
+generate.py:222).  ``--prompt`` is text, or an integer N for a synthetic prompt of N
+random token ids below min(1024, vocabulary) as in generate.py:325-327.  Flags of the
+reference that have no meaning here (--compile, --compile_prefill: the kernels are
+compiled ahead of time) are accepted and ignored; those of features outside this
+library (--interactive, --speculate_k, --draft_checkpoint_path) are refused.
+"""
+import argparse
+import sys
+import time
+from pathlib import Path
+from typing import List, Optional, Union
+
+import torch
+
+from ..config.registry import architecture
+from ..sampling import SamplingParams
+from .generate import generate
+from .step import Engine
+from .tokenizer import encode_tokens, get_tokenizer
+
+
+def _int_or_str(x):
+    try:
+        return int(x)
+    except ValueError:
+        return x
+
+
+def build_parser() -> argparse.ArgumentParser:
+    p = argparse.ArgumentParser(prog="gpt_fast_amd", description="Generate with a Llama model "
+                                "on an MI355X.")
+    p.add_argument("--prompt", type=_int_or_str, default="Hello, my name is",
+                   help="Input prompt. If it's an integer, will instead generate a synthetic prompt.")
+    p.add_argument("--prompt_ids", type=str, default=None,
+                   help="Comma-separated token ids to use as the prompt instead of --prompt.")
+    p.add_argument("--interactive", action="store_true", help="(not available)")
+    p.add_argument("--num_samples", type=int, default=5, help="Number of samples.")
+    p.add_argument("--max_new_tokens", type=int, default=200, help="Maximum number of new tokens.")
+    p.add_argument("--batch_size", type=int, default=1, help="Batch size to benchmark with")
+    p.add_argument("--top_k", type=int, default=200, help="Top-k for sampling.")
+    p.add_argument("--temperature", type=float, default=0.8, help="Temperature for sampling.")
+    p.add_argument("--checkpoint_path", type=Path, default=None,
+                   help="Model folder (config.json and safetensors files).")
+    p.add_argument("--random", type=str, default=None, metavar="PRESET",
+                   help="Use seeded random weights of a named configuration instead of a folder.")
+    p.add_argument("--seed", type=int, default=1234, help="Seed of sampling and of --random.")
+    p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--max_seq_length", type=int, default=None,
+                   help="Cache positions per sequence (default: prompt + new tokens).")
+    p.add_argument("--compile", action="store_true", help="Accepted for compatibility; no effect.")
+    p.add_argument("--compile_prefill", action="store_true",
+                   help="Accepted for compatibility; no effect.")
+    p.add_argument("--profile", type=Path, default=None, help="Profile path.")
+    p.add_argument("--speculate_k", type=int, default=None, help="(not available)")
+    p.add_argument("--draft_checkpoint_path", type=Path, default=None, help="(not available)")
+    p.add_argument("--device", type=str, default="cuda", help="Device to use")
+    return p
+
+
+def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: int = 5,
+         max_new_tokens: int = 100, batch_size: int = 1, top_k: Optional[int] = 200,
+         temperature: float = 0.8, checkpoint_path: Optional[Path] = None,
+         random: Optional[str] = None, seed: int = 1234, dtype: str = "bfloat16",
+         max_seq_length: Optional[int] = None, profile: Optional[Path] = None,
+         device: str = "cuda", out=print) -> dict:
+    """Generates samples and reports throughput the way the reference's ``main`` does
+    (generate.py:272-437).  Returns the aggregate numbers it printed."""
+    if (checkpoint_path is None) == (random is None):
+        raise SystemExit("give either --checkpoint_path MODEL_FOLDER or --random PRESET")
+    device = "cuda:0" if device == "cuda" else device
+    out(f"Using device={device}")
+
+    tokenizer = None
+    if isinstance(prompt, list):
+        encoded = [int(t) for t in prompt]
+    elif isinstance(prompt, int):
+        encoded = None                       # synthetic, needs the vocabulary size
+    else:
+        tokenizer = get_tokenizer(str(checkpoint_path)) if checkpoint_path else None
+        if tokenizer is None:
+            raise SystemExit("a text prompt needs a tokenizer.model or tokenizer.json in the "
+                             "model folder (and sentencepiece or tokenizers); use an integer "
+                             "--prompt for a synthetic prompt, or --prompt_ids")
+        encoded = encode_tokens(tokenizer, prompt, bos=True)
+    prompt_length = prompt if encoded is None else len(encoded)
+    per_seq = max_seq_length or (prompt_length + max_new_tokens)
+    per_seq = (per_seq + 63) // 64 * 64
+    if prompt_length + max_new_tokens > per_seq:
+        raise SystemExit(f"prompt ({prompt_length}) + max_new_tokens ({max_new_tokens}) exceed "
+                         f"--max_seq_length {per_seq}")
+
+    out("Loading model ...")
+    t0 = time.time()
+    cache_args = dict(max_tokens=per_seq * batch_size, max_sequences=batch_size)
+    if random is not None:
+        arch = architecture("llama")
+        engine = Engine.from_random("llama", arch.presets(random), seed, dtype=dtype,
+                                    device=device, **cache_args)
+    else:
+        engine = Engine.from_folder(str(checkpoint_path), dtype=dtype, device=device, **cache_args)
+    torch.cuda.synchronize()
+    out(f"Time to load model: {time.time() - t0:.02f} seconds")
+
+    if encoded is None:
+        g = torch.Generator().manual_seed(seed)
+        hi = min(1024, engine.vocab_size)
+        encoded = torch.randint(0, hi, (prompt,), generator=g).tolist()
+    model_size = engine.model.parameter_bytes()
+    tokens_per_sec = []
+    result = None
+    for i in range(-1, num_samples):                       # sample -1 warms up, generate.py:352
+        torch.cuda.synchronize()
+        prof = None
+        if profile is not None and i == num_samples - 1:
+            prof = torch.profiler.profile()
+            prof.__enter__()
+        t0 = time.perf_counter()
+        result = generate(engine, [encoded] * batch_size, max_new_tokens,
+                          temperature=temperature, top_k=top_k, seed=seed + max(i, 0))
+        torch.cuda.synchronize()
+        t = time.perf_counter() - t0
+        if prof is not None:
+            prof.__exit__(None, None, None)
+            prof.export_chrome_trace(f"{profile}.json")
+        if i == -1:
+            out(f"Warm-up time: {t:.2f} seconds")
+            continue
+        if batch_size > 1:
+            out("Only displaying the first generation of the batch")
+        seq = encoded + result.tokens[0]
+        out(tokenizer.decode(seq) if tokenizer is not None else " ".join(map(str, seq)))
+        generated = len(result.tokens[0])
+        tps = generated / t
+        tokens_per_sec.append(tps)
+        out(f"Time for inference {i + 1}: {t:.02f} sec total, {tps:.02f} tokens/sec")
+        out(f"Bandwidth achieved: {model_size * tps / 1e9:.02f} GB/s")
+        st = result.stats
+        if st.get("decode_steps"):
+            out(f"Decode: {st['decode_steps'] * batch_size / st['decode_seconds']:.02f} tokens/sec "
+                f"over the batch; prefill {st['prefill_seconds'] * 1e3:.1f} ms")
+        out("")
+    out("==========")
+    out(f"Batch Size: {batch_size}")
+    out(f"Prompt Length: {prompt_length}")
+    out(f"Generated tokens: {max_new_tokens}")
+    mean = sum(tokens_per_sec) / max(len(tokens_per_sec), 1)
+    out(f"Average tokens/sec: {mean:.2f}")
+    out(f"Memory used: {torch.cuda.max_memory_reserved() / 1e9:.02f} GB")
+    return {"tokens_per_sec": mean, "result": result}
+
+
+def cli(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    if args.interactive:
+        raise SystemExit("--interactive is not part of this library")
+    if args.speculate_k is not None or args.draft_checkpoint_path is not None:
+        raise SystemExit("speculative decoding is not part of this library")
+    prompt = args.prompt
+    if args.prompt_ids:
+        prompt = [int(t) for t in args.prompt_ids.split(",")]
+    main(prompt, args.num_samples, args.max_new_tokens, args.batch_size, args.top_k,
+         args.temperature, args.checkpoint_path, args.random, args.seed, args.dtype,
+         args.max_seq_length, args.profile, args.device)
+    return 0

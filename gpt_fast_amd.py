@@ -16,3 +16,7 @@ _spec = importlib.util.spec_from_file_location(
 _package = importlib.util.module_from_spec(_spec)
 sys.modules["gpt_fast_amd"] = _package
 _spec.loader.exec_module(_package)
+
+if __name__ == "__main__":          # python -m gpt_fast_amd ...  /  python gpt_fast_amd.py ...
+    from gpt_fast_amd.engine.cli import cli
+    sys.exit(cli())

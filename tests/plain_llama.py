@@ -80,6 +80,8 @@ def read_safetensors(path):
             t = torch.from_numpy(np.frombuffer(buf, dtype="<f2").copy()).float()
         elif dt == "F64":
             t = torch.from_numpy(np.frombuffer(buf, dtype="<f8").copy())
+        elif dt in ("I32", "I64"):
+            t = torch.from_numpy(np.frombuffer(buf, dtype="<i4" if dt == "I32" else "<i8").copy())
         else:
             raise ValueError(f"{name}: dtype {dt}")
         out[name] = t.reshape(shape)

@@ -1,0 +1,228 @@
+"""The cache's bookkeeping and the generation loop's decisions.  No GPU: the cache is
+built on CPU tensors and the loop is driven by a scripted stepper."""
+import random
+
+import pytest
+import torch
+
+from gpt_fast_amd.cache.slots import CacheFull, FreeList
+from gpt_fast_amd.cache.store import Cache, KVNeed, StateNeed
+from gpt_fast_amd.engine.batch import BatchLayout, Entry, fill_host
+from gpt_fast_amd.engine.generate import BatchRun, generate, split_batches
+
+import numpy as np
+
+
+def test_free_list_never_loses_or_doubles():
+    f = FreeList(5, "thing")
+    got = [f.take() for _ in range(5)]
+    assert got == [0, 1, 2, 3, 4] and f.free == 0
+    with pytest.raises(CacheFull):
+        f.take()
+    f.give(3)
+    f.give(1)
+    with pytest.raises(ValueError, match="not held"):
+        f.give(3)                                   # freed twice
+    with pytest.raises(ValueError):
+        f.give(9)
+    assert f.take() == 1 and f.take() == 3          # lowest first: slots are used again
+    f.check()
+    rng = random.Random(0)
+    held = set(range(5))
+    for _ in range(500):
+        if held and rng.random() < 0.5:
+            i = rng.choice(sorted(held))
+            f.give(i)
+            held.remove(i)
+        elif f.free:
+            i = f.take()
+            assert i not in held
+            held.add(i)
+        f.check()
+        assert f.held == len(held)
+
+
+def make_cache(max_tokens=64 * 6, max_sequences=4, window=None):
+    needs = [KVNeed(2, 8, None), KVNeed(2, 8, window), KVNeed(2, 8, None), StateNeed((3,))]
+    return Cache(needs, [None, None, None, None], max_tokens=max_tokens,
+                 max_sequences=max_sequences, dtype=torch.float32, device="cpu")
+
+
+def test_groups_by_need():
+    c = make_cache(window=32)
+    # runs 0 and 2 share a group (equal needs), the windowed run and the state run have their own
+    assert len(c.groups) == 3
+    assert c.entries[0].group_id == c.entries[2].group_id != c.entries[1].group_id
+    assert (c.entries[0].index, c.entries[2].index) == (0, 1)
+    assert c.groups[c.entries[0].group_id].k.shape == (2, 6, 2, 64, 8)
+    assert c.entries[3].state.shape == (4, 3)
+    # a borrowed entry reads the lender's storage and does not write
+    b = Cache([KVNeed(1, 8), KVNeed(1, 8)], [None, 0], max_tokens=64, max_sequences=1,
+              dtype=torch.float32, device="cpu")
+    assert b.entries[1].index == b.entries[0].index and not b.entries[1].writes
+    assert b.groups[0].entries == 1
+
+
+def test_pages_follow_lengths_and_come_back():
+    c = make_cache()
+    a, b = c.acquire(), c.acquire()
+    assert c.extend(a, 70) == 0 and c.length(a) == 70
+    assert len(c.page_list(0, a)) == 2
+    assert c.extend(b, 1) == 0
+    assert c.extend(a, 58) == 70 and len(c.page_list(0, a)) == 2      # 128 tokens: still 2 pages
+    assert c.extend(a, 1) == 128 and len(c.page_list(0, a)) == 3
+    assert c.tokens_held() == 192 + 64
+    c.check()
+    # all-or-nothing: 6 pages in the pool, 4 held; this step would need 3 more
+    with pytest.raises(CacheFull):
+        c.extend_many([(a, 64), (b, 128)])
+    assert c.length(a) == 129 and c.length(b) == 1
+    c.check()
+    pages_a = list(c.page_list(0, a))
+    c.release(a)
+    with pytest.raises(ValueError, match="not held"):
+        c.release(a)
+    with pytest.raises(ValueError):
+        c.extend(a, 1)
+    d = c.acquire()
+    assert d == a and c.length(d) == 0                # the slot is used again
+    c.extend(d, 64 * 3)
+    assert set(c.page_list(0, d)) == set(pages_a)     # and so are its pages
+    c.check()
+    c.release(b)
+    c.release(d)
+    c.check()
+    assert c.slots.held == 0 and all(g.pages.held == 0 for _, g in c.kv_groups)
+
+
+def test_same_slot_twice_in_a_step_is_refused():
+    c = make_cache()
+    a = c.acquire()
+    with pytest.raises(ValueError, match="twice"):
+        c.extend_many([(a, 1), (a, 1)])
+    with pytest.raises(ValueError):
+        c.extend(a, 0)
+
+
+def test_window_gives_pages_back():
+    c = make_cache(max_tokens=64 * 8, window=70)
+    wg = c.entries[1].group_id
+    a = c.acquire()
+    c.extend(a, 64 * 4)
+    assert c.groups[wg].pages.held == 4
+    c.extend(a, 1)            # start = 256: keys below 256 - 70 + 1 = 187 are out of reach
+    assert c.page_list(wg, a)[:2] == [-1, -1] and c.page_list(wg, a)[2] >= 0
+    assert c.groups[wg].pages.held == 3
+    assert c.groups[c.entries[0].group_id].pages.held == 5      # the full group keeps all
+    c.check()
+    c.release(a)
+    c.check()
+
+
+def test_state_is_zeroed_at_acquire():
+    c = make_cache()
+    a = c.acquire()
+    c.entries[3].state[a] += 5.0
+    c.release(a)
+    assert c.acquire() == a
+    assert float(c.entries[3].state[a].abs().sum()) == 0.0
+
+
+def test_batch_description_layout():
+    c = make_cache()
+    a, b = c.acquire(), c.acquire()
+    starts = c.extend_many([(a, 3), (b, 70)])
+    entries = [Entry(a, [5, 6, 7], want=[0, 2], key=11), Entry(b, list(range(70)), want=[69], key=12)]
+    widths = {gid: 2 for gid, _ in c.kv_groups}
+    lay = BatchLayout(73, 2, 3, widths)
+    host = np.zeros(lay.size, dtype=np.int32)
+    fill_host(lay, host, entries, starts, c)
+    f = lambda name: host[lay.fields[name][0]: lay.fields[name][0] + lay.fields[name][1]]
+    assert list(f("tokens")[:4]) == [5, 6, 7, 0]
+    assert list(f("tok_seq")[:4]) == [0, 0, 0, 1] and list(f("tok_pos")[:5]) == [0, 1, 2, 0, 1]
+    assert list(f("q_start")) == [0, 3, 73] and list(f("want_rows")) == [0, 2, 72]
+    assert list(f("row_keys")) == [11, 12]
+    off, n = lay.tables[0]
+    table = host[off:off + n].reshape(2, 2)
+    assert table[0, 0] == c.page_list(0, a)[0] and table[0, 1] == -1
+    assert list(table[1]) == c.page_list(0, b)
+    with pytest.raises(ValueError):
+        fill_host(lay, host, [Entry(a, [1, 2, 3], want=[3]), entries[1]], starts, c)
+
+
+class ScriptedStepper:
+    """Hands out slots, checks what the loop asks for, answers from a script:
+    the token for (request key, number of tokens fed so far)."""
+
+    def __init__(self, script, n_slots=8):
+        self.script = script
+        self.slots = FreeList(n_slots, "slot")
+        self.fed = {}
+        self.calls = []
+
+    def start_sequence(self):
+        s = self.slots.take()
+        self.fed[s] = []
+        return s
+
+    def end_sequence(self, slot):
+        self.slots.give(slot)
+        del self.fed[slot]
+
+    def next_tokens(self, entries):
+        out = []
+        self.calls.append([(e.key, list(e.tokens)) for e in entries])
+        for e in entries:
+            assert list(e.want) == [len(e.tokens) - 1]
+            self.fed[e.slot] += list(e.tokens)
+            out.append(self.script(e.key, self.fed[e.slot]))
+        return out
+
+
+def test_loop_unequal_prompts_stop_tokens_and_early_ends():
+    # every request echoes (last token + 1); token 50 is the stop token
+    st = ScriptedStepper(lambda key, fed: fed[-1] + 1)
+    prompts = [[10, 11], [47], [30, 31, 32], [49]]
+    run = BatchRun(st, prompts, keys=[0, 1, 2, 3], max_new_tokens=5, stop_tokens=[50])
+    new, why = run.run()
+    assert new == [[12, 13, 14, 15, 16], [48, 49, 50], [33, 34, 35, 36, 37], [50]]
+    assert why == ["length", "stop", "length", "stop"]
+    # the prompts go in one step, then one token per live request; ended ones drop out
+    assert st.calls[0] == [(0, [10, 11]), (1, [47]), (2, [30, 31, 32]), (3, [49])]
+    assert st.calls[1] == [(0, [12]), (1, [48]), (2, [33])]
+    assert st.calls[3] == [(0, [14]), (2, [35])]
+    assert len(st.calls) == 5 and run.steps == 5      # reference: max_new_tokens model calls
+    assert st.slots.held == 0
+
+
+def test_loop_gives_slots_back_on_errors():
+    def script(key, fed):
+        if len(fed) > 3:
+            raise RuntimeError("boom")
+        return 1
+    st = ScriptedStepper(script)
+    with pytest.raises(RuntimeError):
+        BatchRun(st, [[1], [2, 3]], [0, 1], 9).run()
+    assert st.slots.held == 0
+    with pytest.raises(ValueError):
+        BatchRun(st, [[]], [0], 3)
+    with pytest.raises(ValueError):
+        BatchRun(st, [[1]], [0], 0)
+
+
+def test_batches_one_after_another_reuse_slots():
+    assert split_batches(5, 2) == [[0, 1], [2, 3], [4]]
+    assert split_batches(3, None) == [[0, 1, 2]] and split_batches(0, 4) == []
+    st = ScriptedStepper(lambda key, fed: key, n_slots=2)
+
+    class FakeEngine:
+        class model:
+            class plan:
+                stop_tokens = ()
+    seen = []
+    res = generate(FakeEngine, [[1], [2, 2], [3], [4, 4, 4], [5]], 3, temperature=0.0,
+                   batch_size=2, stepper=st, callback=lambda rows, toks: seen.append((rows, toks)))
+    assert res.tokens == [[0] * 3, [1] * 3, [2] * 3, [3] * 3, [4] * 3]
+    assert res.finish_reasons == ["length"] * 5 and res.stats["steps"] == 9
+    assert seen[0] == ([0, 1], [0, 1]) and seen[3] == ([2, 3], [2, 3]) and seen[-1] == ([4], [4])
+    assert st.slots.held == 0

@@ -1,0 +1,193 @@
+"""Configuration, registry, safetensors reading, weight errors and the random-weights
+mode.  No GPU."""
+import json
+import os
+
+import pytest
+import torch
+
+import plain_llama as plain
+import util
+
+import gpt_fast_amd as gfa
+from gpt_fast_amd.config.llama import ConfigError, LlamaConfig, preset_dict
+from gpt_fast_amd.config.registry import UnknownArchitecture, architecture_of
+from gpt_fast_amd.weights.bindings import WeightsError, load_parameters
+from gpt_fast_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+
+
+def test_config_from_keys_and_derivations():
+    c = LlamaConfig.from_dict(util.TINY_B)
+    assert (c.hidden_size, c.num_attention_heads, c.num_key_value_heads, c.head_dim) == (192, 6, 2, 32)
+    assert c.intermediate_size == 512 and c.rms_norm_eps == 1e-6 and c.rope_theta == 500000.0
+    assert dict(c.rope_scaling)["original_max_position_embeddings"] == 32
+    # derived values of the reference (model.py:36-42)
+    d = LlamaConfig.from_dict(dict(hidden_size=4096, num_attention_heads=32,
+                                   num_hidden_layers=2, vocab_size=100))
+    assert d.num_key_value_heads == 32 and d.head_dim == 128 and d.intermediate_size == 11008
+    # a given intermediate_size and head_dim are honoured
+    assert LlamaConfig.from_dict(util.TINY_A).intermediate_size == 176
+    assert LlamaConfig.from_dict(util.TINY_C).head_dim == 48
+    # round trip through config.json keys
+    assert LlamaConfig.from_dict(c.to_dict()) == c
+
+
+def test_presets_match_reference_registry():          # model.py:44-82
+    c = LlamaConfig.from_name("llama-3.1-8b")
+    assert (c.num_hidden_layers, c.hidden_size, c.intermediate_size, c.vocab_size) == (32, 4096, 14336, 128256)
+    assert dict(c.rope_scaling)["factor"] == 8.0 and c.max_position_embeddings == 131072
+    # fuzzy match: longest preset name contained in the given name wins
+    assert LlamaConfig.from_name("Meta-Llama-3.1-70B-Instruct").num_hidden_layers == 80
+    assert LlamaConfig.from_name("Mistral-7B-v0.1").num_key_value_heads == 8
+    assert LlamaConfig.from_name("llama-2-7b-chat-hf").intermediate_size == 11008
+    with pytest.raises(ConfigError):
+        LlamaConfig.from_name("nothing-like-it")
+
+
+@pytest.mark.parametrize("patch,word", [
+    ({"attention_bias": True}, "attention_bias"), ({"mlp_bias": True}, "mlp_bias"),
+    ({"hidden_act": "gelu"}, "hidden_act"), ({"rope_scaling": {"rope_type": "yarn"}}, "yarn"),
+    ({"num_key_value_heads": 3}, "multiple"), ({"head_dim": 15}, "even"),
+    ({"hidden_size": None}, "hidden_size"),
+])
+def test_config_refusals(patch, word):
+    raw = dict(util.TINY_A)
+    raw.update(patch)
+    with pytest.raises(ConfigError, match=word):
+        LlamaConfig.from_dict(raw)
+
+
+def test_registry_names_the_model():
+    assert architecture_of({"architectures": ["LlamaForCausalLM"]}) is gfa.architecture("llama")
+    assert architecture_of({"model_type": "llama"}) is gfa.architecture("LlamaForCausalLM")
+    with pytest.raises(UnknownArchitecture, match="LlamaForCausalLM"):
+        architecture_of({"architectures": ["SomethingElse"]})
+    with pytest.raises(UnknownArchitecture):
+        architecture_of({})
+
+
+def test_plan_is_data():
+    arch = gfa.architecture("llama")
+    plan = arch.plan(LlamaConfig.from_dict(util.TINY_B))
+    assert len(plan.layers) == 3 and [r.layer for r in plan.order] == [0, 1, 2]
+    m = plan.layers[1].mixer
+    assert (m.n_heads, m.n_kv_heads, m.head_dim, m.position.base) == (6, 2, 32, 500000.0)
+    assert plan.layers[0].mixer_norm.eps == 1e-6 and plan.layers[2].feed_forward.hidden == 512
+
+
+def test_safetensors_round_trip(tmp_path):
+    t = {"a": torch.randn(3, 5), "b": torch.randn(7).to(torch.bfloat16),
+         "c": torch.arange(6, dtype=torch.int32).reshape(2, 3)}
+    path = str(tmp_path / "x.safetensors")
+    write_safetensors(path, t)
+    f = SafetensorsFile(path)
+    assert f.entries["b"] == ("BF16", (7,))
+    for k, v in t.items():
+        assert torch.equal(f.tensor(k), v)
+    # the plain reader and the safetensors package read the same file
+    mine = plain.read_safetensors(path)
+    assert torch.equal(mine["a"], t["a"]) and torch.equal(mine["b"], t["b"].float())
+    from safetensors.torch import load_file
+    theirs = load_file(path)
+    assert all(torch.equal(theirs[k], v) for k, v in t.items())
+
+
+def _folder(tmp_path, name="A", dtype="float32"):
+    return util.make_folder(tmp_path, name, seed=1, dtype=dtype)
+
+
+def test_loader_fuses_and_permutes_like_the_converter(tmp_path):
+    folder = _folder(tmp_path, "B")
+    arch, cfg = gfa.read_model_folder(folder)
+    params = load_parameters(folder, arch.bindings(cfg), "float32", None)
+    pcfg, w = plain.load_folder(folder)
+    assert torch.equal(params["layers.1.attention.wqkv"], w["layers.1.attention.wqkv.weight"])
+    assert torch.equal(params["layers.2.feed_forward.w13"][:512], w["layers.2.feed_forward.w1.weight"])
+    assert torch.equal(params["layers.2.feed_forward.w13"][512:], w["layers.2.feed_forward.w3.weight"])
+    assert params["norm.weight"].dtype == torch.float32
+
+
+def test_loader_dtypes(tmp_path):
+    folder = _folder(tmp_path, "A", dtype="bfloat16")
+    arch, cfg = gfa.read_model_folder(folder)
+    p = load_parameters(folder, arch.bindings(cfg), "bfloat16", None)
+    assert p["layers.0.attention.wo"].dtype == torch.bfloat16          # matrices: compute type
+    assert p["layers.0.ffn_norm.weight"].dtype == torch.float32         # vectors: 32-bit
+    p32 = load_parameters(folder, arch.bindings(cfg), "float32", None)
+    assert p32["layers.0.attention.wo"].dtype == torch.float32
+    assert torch.equal(p32["layers.0.attention.wo"], p["layers.0.attention.wo"].float())
+
+
+def test_tied_embeddings(tmp_path):
+    folder = _folder(tmp_path, "C")
+    names = SafetensorsFile(os.path.join(folder, "model.safetensors")).entries
+    assert "lm_head.weight" not in names
+    arch, cfg = gfa.read_model_folder(folder)
+    p = load_parameters(folder, arch.bindings(cfg), "float32", None)
+    assert p["output.weight"].data_ptr() == p["tok_embeddings.weight"].data_ptr()
+
+
+def test_one_error_lists_everything(tmp_path):
+    folder = _folder(tmp_path, "A")
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {k: f.tensor(k).clone() for k in f.entries}
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(32, 64)
+    tensors["model.layers.7.extra.weight"] = torch.zeros(2)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)     # ignored
+    bad = str(tmp_path / "bad")
+    os.makedirs(bad)
+    write_safetensors(os.path.join(bad, "model.safetensors"), tensors)
+    with open(os.path.join(bad, "config.json"), "w") as g:
+        json.dump(util.TINY_A, g)
+    arch, cfg = gfa.read_model_folder(bad)
+    with pytest.raises(WeightsError) as e:
+        load_parameters(bad, arch.bindings(cfg), "float32", None)
+    err = e.value
+    assert err.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.7.extra.weight"]
+    assert err.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 64), (64, 64))]
+    text = str(err)
+    for word in ("missing", "unexpected", "wrong shapes", "up_proj", "extra", "[32, 64]"):
+        assert word in text
+
+
+def test_missing_files(tmp_path):
+    with pytest.raises(FileNotFoundError, match="config.json"):
+        gfa.read_model_folder(str(tmp_path))
+    with open(tmp_path / "config.json", "w") as g:
+        json.dump(util.TINY_A, g)
+    arch, cfg = gfa.read_model_folder(str(tmp_path))
+    with pytest.raises(FileNotFoundError, match="model.safetensors"):
+        load_parameters(str(tmp_path), arch.bindings(cfg), "float32", None)
+
+
+def test_random_model_is_seeded_and_sharded_index_is_read(tmp_path):
+    a = util.make_folder(tmp_path / "x", "A", seed=5)
+    b = util.make_folder(tmp_path / "y", "A", seed=5)
+    c = util.make_folder(tmp_path / "z", "A", seed=6)
+    fa, fb, fc = (SafetensorsFile(os.path.join(f, "model.safetensors")) for f in (a, b, c))
+    name = "model.layers.1.self_attn.q_proj.weight"
+    assert torch.equal(fa.tensor(name), fb.tensor(name))
+    assert not torch.equal(fa.tensor(name), fc.tensor(name))
+    norm = fa.tensor("model.layers.0.input_layernorm.weight")
+    assert abs(float(norm.mean()) - 1.0) < 0.1                  # 1 + N(0, 0.1)
+    cfg = json.load(open(os.path.join(a, "config.json")))
+    assert cfg["architectures"] == ["LlamaForCausalLM"] and cfg["hidden_size"] == 64
+    # split into two shards with an index file
+    tensors = {k: fa.tensor(k).clone() for k in fa.entries}
+    keys = sorted(tensors)
+    sh = str(tmp_path / "sharded")
+    os.makedirs(sh)
+    write_safetensors(os.path.join(sh, "m-1.safetensors"), {k: tensors[k] for k in keys[:5]})
+    write_safetensors(os.path.join(sh, "m-2.safetensors"), {k: tensors[k] for k in keys[5:]})
+    index = {"weight_map": {k: ("m-1.safetensors" if i < 5 else "m-2.safetensors")
+                            for i, k in enumerate(keys)}}
+    json.dump(index, open(os.path.join(sh, "model.safetensors.index.json"), "w"))
+    json.dump(cfg, open(os.path.join(sh, "config.json"), "w"))
+    arch, c2 = gfa.read_model_folder(sh)
+    p1 = load_parameters(sh, arch.bindings(c2), "float32", None)
+    p0 = load_parameters(a, arch.bindings(c2), "float32", None)
+    assert all(torch.equal(p0[k], p1[k]) for k in p0)

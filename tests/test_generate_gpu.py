@@ -1,0 +1,326 @@
+"""Generation through the entry points, trace replay as a program, parts alone, and a
+toy mixer with state of its own that is registered from here."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as plain
+import util
+from util import TOL_BF16, TOL_F32, rel_err
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def engine_for(folder, dtype, **kw):
+    import gpt_fast_amd as gfa
+    kw.setdefault("max_tokens", 4096)
+    return gfa.Engine.from_folder(folder, dtype=dtype, device="cuda:0", **kw)
+
+
+@pytest.mark.parametrize("name,prompt_lens,new", [("A", [7, 3, 12], 8), ("B", [1, 5, 17, 33], 16)])
+def test_greedy_generation_equals_plain(tmp_path_factory, name, prompt_lens, new):
+    import gpt_fast_amd as gfa
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name)
+    cfg, w = plain.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 40 + n) for n in prompt_lens]
+    want = [plain.greedy_generate(w, cfg, p, new) for p in prompts]
+    eng = engine_for(folder, "float32")
+    res = gfa.generate(eng, prompts, max_new_tokens=new, temperature=0.0)
+    assert res.tokens == want
+    assert res.finish_reasons == ["length"] * len(prompts)
+    assert eng.cache.slots.held == 0
+    # one request alone gives the same tokens as in the batch; so do smaller batches
+    alone = gfa.generate(eng, prompts[1:2], max_new_tokens=new, temperature=0.0)
+    assert alone.tokens == want[1:2]
+    two = gfa.generate(eng, prompts, max_new_tokens=new, temperature=0.0, batch_size=2)
+    assert two.tokens == want
+    # bfloat16: tokens agree wherever the float32 decision was not close
+    eb = engine_for(folder, "bfloat16")
+    got = gfa.generate(eb, prompts, max_new_tokens=new, temperature=0.0).tokens
+    for p, g, wnt in zip(prompts, got, want):
+        for i, (a, b) in enumerate(zip(g, wnt)):
+            if a != b:
+                logits = plain.forward(w, cfg, p + wnt[:i])[-1]
+                top = torch.topk(logits, 2).values
+                assert float(top[0] - top[1]) < 0.05 * float(logits.abs().max()), (i, a, b)
+                break
+
+
+def test_stop_tokens_end_only_their_sequence(tmp_path_factory):
+    import gpt_fast_amd as gfa
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "A")
+    cfg, w = plain.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 70 + n) for n in (4, 9, 6)]
+    free = [plain.greedy_generate(w, cfg, p, 10) for p in prompts]
+    stop = free[1][3]                          # the 4th token of request 1 becomes a stop token
+    want = [plain.greedy_generate(w, cfg, p, 10, stop_tokens=(stop,)) for p in prompts]
+    assert len(want[1]) <= 4
+    eng = engine_for(folder, "float32")
+    res = gfa.generate(eng, prompts, max_new_tokens=10, temperature=0.0, stop_tokens=[stop])
+    assert res.tokens == want
+    assert res.finish_reasons[1] == "stop" and res.tokens[1][-1] == stop
+    assert eng.cache.slots.held == 0
+
+
+def test_sampled_generation_is_seeded_and_batch_independent(tmp_path_factory):
+    import gpt_fast_amd as gfa
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg = plain.read_config(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 90 + n) for n in (1, 5, 17, 33)]
+    eng = engine_for(folder, "float32")
+    kw = dict(max_new_tokens=16, temperature=0.8, top_k=50)
+    a = gfa.generate(eng, prompts, seed=7, **kw).tokens
+    b = gfa.generate(eng, prompts, seed=7, **kw).tokens
+    c = gfa.generate(eng, prompts, seed=8, **kw).tokens
+    assert a == b and a != c
+    assert all(len(t) == 16 for t in a)
+    # the same requests in batches of two draw the same tokens (noise is per request)
+    d = gfa.generate(eng, prompts, seed=7, batch_size=2, **kw).tokens
+    assert d == a
+
+
+def test_long_decoding_and_first_tokens(tmp_path_factory):
+    """300 tokens decoded one by one from a one-token prompt: the first tokens of a
+    sequence, page edges at 64, 128, 192, 256, and a long run, float32 and bfloat16."""
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg, w = plain.load_folder(folder)
+    tokens = util.random_tokens(cfg["vocab"], 300, 5)
+    want = plain.forward(w, cfg, tokens)
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        eng = engine_for(folder, dtype)
+        slot = eng.start_sequence()
+        got = torch.cat([eng.step([Entry(slot, [t], want=[0])]).cpu() for t in tokens])
+        eng.end_sequence(slot)
+        assert rel_err(got[:4], want[:4]) < tol
+        assert rel_err(got, want) < tol
+
+
+def test_decode_session_with_graph_equals_stepping(tmp_path_factory):
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.engine.decode import DecodeSession
+    from gpt_fast_amd.sampling import SamplingParams
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg, w = plain.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 20 + n) for n in (60, 3, 64)]
+    want = [plain.greedy_generate(w, cfg, p, 12) for p in prompts]
+    for use_graph in (False, True):
+        eng = engine_for(folder, "float32")
+        slots = [eng.start_sequence() for _ in prompts]
+        logits = eng.step([Entry(s, p, want=[len(p) - 1]) for s, p in zip(slots, prompts)])
+        first = logits.argmax(-1).to(torch.int32)
+        sess = DecodeSession(eng, slots, [0, 1, 2], first, SamplingParams(temperature=0.0),
+                             use_graph=use_graph, max_new_tokens=12)
+        got = [first.cpu()]
+        for _ in range(11):
+            got.append(sess.advance().cpu().clone())       # crosses a page edge at 64
+            torch.cuda.synchronize()
+        got = torch.stack(got, 1).tolist()
+        assert got == want, use_graph
+        for s in slots:
+            eng.end_sequence(s)
+
+
+def _replay(folder, dtype, steps, out, max_tokens):
+    lines = "\n".join(json.dumps(s) for s in steps) + "\n"
+    env = dict(os.environ)
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", out, "--max-tokens", str(max_tokens)],
+                          input=lines, capture_output=True, text=True, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == \
+        [f"done {s['step']}" for s in steps]
+
+
+def test_trace_run_program(tmp_path_factory, tmp_path):
+    """bin/trace_run on a trace of two batches of unequal requests; the second batch reuses
+    what the first gave back; max-tokens is exactly what the live requests hold."""
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "C")
+    cfg, w = plain.load_folder(folder)
+    V = cfg["vocab"]
+    reqs = {"a": util.random_tokens(V, 70, 1), "b": util.random_tokens(V, 5, 2),
+            "c": util.random_tokens(V, 130, 3), "d": util.random_tokens(V, 64, 4)}
+    prompt = {"a": 66, "b": 2, "c": 128, "d": 60}
+    steps = []
+    where = {}                                  # request -> list of (step, first row, count)
+
+    def batch(ids, n0):
+        n = n0
+        live = list(ids)
+        steps.append({"step": n, "entries": [
+            {"id": r, "tokens": reqs[r][:prompt[r]], "want": list(range(prompt[r]))} for r in live],
+            "end": []})
+        at = 0
+        for r in live:
+            where.setdefault(r, []).append((n, at, prompt[r]))
+            at += prompt[r]
+        t = 0
+        while live:
+            n += 1
+            ending = [r for r in live if prompt[r] + t + 1 >= len(reqs[r])]
+            steps.append({"step": n, "entries": [
+                {"id": r, "tokens": [reqs[r][prompt[r] + t]], "want": [0]} for r in live],
+                "end": ending})
+            for row, r in enumerate(live):
+                where[r].append((n, row, 1))
+            live = [r for r in live if r not in ending]
+            t += 1
+        return n + 1
+
+    n = batch(["a", "b"], 0)
+    batch(["c", "d"], n)
+    most = max(128 + 64, 192 + 64)              # a+b: 128+64; c+d: 192+64 tokens in pages
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        out = str(tmp_path / dtype)
+        _replay(folder, dtype, steps, out, most)
+        for r, toks in reqs.items():
+            rows = []
+            for step, row, count in where[r]:
+                data = np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, V)
+                rows.append(torch.from_numpy(data[row:row + count].copy()))
+            got = torch.cat(rows)
+            assert got.shape[0] == len(toks)
+            assert rel_err(got, plain.forward(w, cfg, toks)) < tol, (dtype, r)
+
+
+def test_parts_alone(tmp_path_factory):
+    """Each part of a layer on its own against the plain function of the same part."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.config.spec import GatedFeedForwardSpec, NormSpec
+    from gpt_fast_amd.parts import FEED_FORWARDS, MIXERS, NORMS, Runtime
+    from gpt_fast_amd.cache.store import Cache
+    from gpt_fast_amd.engine.batch import BatchUploader
+    rt = Runtime(torch.float32, "cuda:0")
+    torch.manual_seed(0)
+    D = 72
+    x = torch.randn(9, D, device="cuda:0")
+    # norm
+    norm = NORMS.build(NormSpec(D, 1e-4), rt)
+    wn = torch.randn(D, device="cuda:0")
+    norm.bind({"weight": wn})
+    assert rel_err(norm.forward(x), plain.rms_norm(x.cpu(), wn.cpu(), 1e-4)) < 1e-6
+    # feed-forward adds into the residual stream
+    ff = FEED_FORWARDS.build(GatedFeedForwardSpec(D, 104), rt)
+    w13, w2 = torch.randn(208, D, device="cuda:0") * 0.1, torch.randn(D, 104, device="cuda:0") * 0.1
+    ff.bind({"w13": w13, "w2": w2})
+    res = torch.ones(9, D, device="cuda:0")
+    ff.forward(x, None, res)
+    want = 1 + plain.feed_forward(x.cpu(), w13[:104].cpu(), w13[104:].cpu(), w2.cpu())
+    assert rel_err(res, want) < 1e-5
+    # attention mixer over its own cache entry, prompt then one token
+    arch = gfa.architecture("llama")
+    plan = arch.plan(arch.read_config(util.TINY_B))
+    spec = plan.layers[0].mixer
+    att = MIXERS.build(spec, rt)
+    Dm = spec.dim
+    wqkv = torch.randn((spec.n_heads + 2 * spec.n_kv_heads) * spec.head_dim, Dm, device="cuda:0") * 0.1
+    wo = torch.randn(Dm, spec.n_heads * spec.head_dim, device="cuda:0") * 0.1
+    att.bind({"wqkv": wqkv, "wo": wo})
+    cache = Cache([att.cache_need()], [None], max_tokens=128, max_sequences=2,
+                  dtype=torch.float32, device="cuda:0")
+    up = BatchUploader("cuda:0")
+    xs = torch.randn(70, Dm, device="cuda:0")
+    slot = cache.acquire()
+    res = torch.zeros(70, Dm, device="cuda:0")
+    starts = cache.extend_many([(slot, 69)])
+    att.forward(xs[:69].contiguous(), up.build([Entry(slot, [0] * 69)], starts, cache),
+                cache.entries[0], res[:69])
+    starts = cache.extend_many([(slot, 1)])
+    att.forward(xs[69:].contiguous(), up.build([Entry(slot, [0])], starts, cache),
+                cache.entries[0], res[69:])
+    pcfg = plain.config_from_dict(util.TINY_B)
+    want = plain.attention(xs.cpu(), wqkv.cpu(), wo.cpu(), pcfg, torch.arange(70))
+    assert rel_err(res, want) < 1e-5
+
+
+def test_toy_mixer_with_state_registers_and_steps(tmp_path_factory):
+    """A mixer defined here, with fixed-size state per sequence and no keys or values, is
+    registered, built into a plan next to attention layers, and stepped: no file of the
+    library changes.  It computes a running mean of its inputs (state: sum and count),
+    which the plain check below recomputes from the whole sequence."""
+    from dataclasses import dataclass
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.cache.store import StateNeed
+    from gpt_fast_amd.config.spec import LayerSpec, ModelPlan, NormSpec, Run
+    from gpt_fast_amd.parts import Param, Part, register_mixer
+
+    @dataclass(frozen=True)
+    class RunningMeanSpec:
+        dim: int
+        kind: str = "toy_running_mean"
+
+    class RunningMean(Part):
+        def __init__(self, spec, rt):
+            self.spec, self.rt = spec, rt
+
+        def parameters(self):
+            return {"mix": Param((self.spec.dim, self.spec.dim))}
+
+        def bind(self, tensors):
+            self.mix = tensors["mix"]
+
+        def cache_need(self):
+            return StateNeed((self.spec.dim + 1,), "float32")
+
+        def forward(self, x, batch, entry, residual):
+            state = entry.state                                   # [n_slots, dim + 1]
+            q_start = batch.host_field("q_start")
+            slots = batch.host_field("slots")
+            for b in range(batch.n_seqs):
+                lo, hi = int(q_start[b]), int(q_start[b + 1])
+                xs = x[lo:hi].float()
+                s = state[int(slots[b])]
+                sums = s[:-1] + torch.cumsum(xs, 0)
+                counts = s[-1] + torch.arange(1, hi - lo + 1, device=x.device)
+                residual[lo:hi] += (sums / counts[:, None]) @ self.mix.float().T
+                s[:-1] = sums[-1]
+                s[-1] = counts[-1]
+
+    register_mixer("toy_running_mean", RunningMean)
+
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_A)
+    base = arch.plan(cfg)
+    D = cfg.hidden_size
+    toy_layer = LayerSpec(name="toy", mixer=RunningMeanSpec(D), mixer_norm=NormSpec(D, 1e-5),
+                          feed_forward=base.layers[0].feed_forward,
+                          feed_forward_norm=NormSpec(D, 1e-5))
+    # attention, toy, attention again with the first run's weights *and* cache (borrowed)
+    plan = ModelPlan(dim=D, vocab_size=cfg.vocab_size,
+                     layers=[base.layers[0], toy_layer, base.layers[1]],
+                     order=[Run(0), Run(1), Run(2), Run(1), Run(0, cache_from=0)],
+                     final_norm=base.final_norm)
+    from gpt_fast_amd.parts import Runtime
+    from gpt_fast_amd.parts.model import DecoderModel
+    model = DecoderModel(plan, Runtime(torch.float32, "cuda:0"))
+    g = torch.Generator().manual_seed(0)
+    params = {}
+    for name, p in model.parameters().items():
+        t = torch.randn(p.shape, generator=g) * 0.05
+        params[name] = (1 + t if p.init == "norm" else t).to("cuda:0")
+    eng = gfa.Engine.from_plan(plan, params, "float32", "cuda:0", max_tokens=512)
+    assert len(eng.cache.groups) == 2             # one KV group, one state group of two entries
+    toks = util.random_tokens(cfg.vocab_size, 90, 3)
+    slot = eng.start_sequence()
+    whole = eng.step([Entry(slot, toks, want=list(range(90)))]).cpu()
+    eng.end_sequence(slot)
+    # the same tokens cut into a prompt and single tokens, next to another sequence, in a
+    # slot that was used before: state must have been reset and carried correctly
+    s1, s2 = eng.start_sequence(), eng.start_sequence()
+    other = util.random_tokens(cfg.vocab_size, 40, 4)
+    out = [eng.step([Entry(s1, other[:30]), Entry(s2, toks[:50], want=list(range(50)))]).cpu()]
+    for i in range(50, 90):
+        entries = [Entry(s2, [toks[i]], want=[0])]
+        if i < 60:
+            entries.insert(0, Entry(s1, [other[i - 20]]))
+        out.append(eng.step(entries).cpu())
+    assert rel_err(torch.cat(out), whole) < 1e-5
+    assert not torch.isnan(whole).any() and float(whole.abs().max()) > 0

@@ -1,0 +1,303 @@
+"""Each HIP kernel alone against a plain PyTorch float32 computation of the same op, at
+sizes other than the engine tests' (head sizes in steps of 16, widths and vocabularies
+that are no power of two, odd row counts)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def K():
+    from gpt_fast_amd.ops import kernels
+    return kernels
+
+
+def bf(t):
+    return t.to(torch.bfloat16)
+
+
+def close(a, b, tol):
+    a, b = a.double().cpu(), b.double().cpu()
+    err = float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+    assert err < tol, err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    torch.manual_seed(0)
+    table = torch.randn(333, 72, device=DEV).to(dtype)
+    tok = torch.tensor([0, 332, 5, 5, 17], dtype=torch.int32, device=DEV)
+    assert torch.equal(K().embed(table, tok), table[tok.long()].float())
+
+
+@pytest.mark.parametrize("dim,eps", [(72, 1e-5), (200, 1e-6), (4096, 1e-5), (1000, 0.3)])
+def test_rmsnorm(dim, eps):
+    torch.manual_seed(1)
+    x = torch.randn(7, dim, device=DEV) * 3
+    w = torch.randn(dim, device=DEV)
+    ref = x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()
+    close(K().rmsnorm(x, w, eps, torch.float32), ref, 2e-6)
+    close(K().rmsnorm(x, w, eps, torch.bfloat16), ref, 1e-2)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(K().rmsnorm(x, w, eps, torch.float32, rows=rows),
+                       K().rmsnorm(x, w, eps, torch.float32)[rows.long()])
+    # eps inside the root: it dominates a tiny input
+    tiny = torch.full((1, dim), 1e-4, device=DEV)
+    out = K().rmsnorm(tiny, torch.ones(dim, device=DEV), 1e-2, torch.float32)
+    close(out, tiny / math.sqrt(1e-8 + 1e-2), 1e-5)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 5, 3), (3, 100, 70), (65, 130, 257), (200, 64, 1000)])
+def test_gemm_f32(M, N, K_):
+    torch.manual_seed(2)
+    a = torch.randn(M, K_, device=DEV)
+    w = torch.randn(N, K_, device=DEV)
+    ref = a.double() @ w.double().T
+    out = K().gemm_f32(a, w)
+    close(out, ref, 1e-5)
+    # rows do not depend on the other rows: a float32 result is the same for any cutting
+    assert torch.equal(K().gemm_f32(a[M // 2:M // 2 + 1], w), out[M // 2:M // 2 + 1])
+    res = torch.randn(M, N, device=DEV)
+    keep = res.clone()
+    K().gemm_f32(a, w, out=res, accumulate=True)
+    close(res, keep.double() + ref, 1e-5)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 17, 33, 64])
+@pytest.mark.parametrize("N,K_", [(40, 64), (136, 200), (1000, 328), (96, 4096), (77, 75)])
+def test_skinny_bf16(M, N, K_):
+    from gpt_fast_amd.ops import gemm_bf16 as G
+    torch.manual_seed(3)
+    x = bf(torch.randn(M, K_, device=DEV))
+    w = bf(torch.randn(N, K_, device=DEV) * 0.1)
+    ref = x.double() @ w.double().T
+    close(G.skinny(x, w, out_dtype=torch.float32), ref, 2e-5)
+    close(G.skinny(x, w, out_dtype=torch.bfloat16), ref, 1e-2)
+    res = torch.randn(M, N, device=DEV)
+    keep = res.clone()
+    G.skinny(x, w, residual=res)
+    close(res, keep.double() + ref, 2e-5)
+    close(K().gemm_bf16_naive(x, w), ref, 2e-5)
+    if N % 2 == 0:
+        I = N // 2
+        g = ref[:, :I]
+        close(G.skinny_gated(x, w), (g * torch.sigmoid(g)) * ref[:, I:], 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul_and_add_into(dtype):
+    torch.manual_seed(4)
+    gu = torch.randn(5, 2 * 37, device=DEV).to(dtype)
+    ref = torch.nn.functional.silu(gu[:, :37].double()) * gu[:, 37:].double()
+    close(K().silu_mul(gu), ref, 1e-6 if dtype == torch.float32 else 1e-2)
+    res = torch.randn(5, 37, device=DEV)
+    y = torch.randn(5, 37, device=DEV).to(dtype)
+    want = res + y.float()
+    assert torch.equal(K().add_into(res, y), want)
+
+
+def _paged(S_list, G, hd, dtype, seed):
+    """Random keys/values for sequences of the given lengths scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum((s + 63) // 64 for s in S_list) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    k_pages = torch.full((n_pages, G, 64, hd), float("nan")).to(dtype)      # poison: never read
+    v_pages = torch.full((n_pages, G, 64, hd), float("nan")).to(dtype)
+    width = max((s + 63) // 64 for s in S_list)
+    table = torch.full((len(S_list), width), -1, dtype=torch.int32)
+    ks, vs = [], []
+    for b, S in enumerate(S_list):
+        k = torch.randn(S, G, hd, generator=g).to(dtype)
+        v = torch.randn(S, G, hd, generator=g).to(dtype)
+        ks.append(k)
+        vs.append(v)
+        for i in range((S + 63) // 64):
+            p = perm.pop()
+            table[b, i] = p
+            n = min(64, S - 64 * i)
+            k_pages[p, :, :n] = k[64 * i:64 * i + n].transpose(0, 1)
+            v_pages[p, :, :n] = v[64 * i:64 * i + n].transpose(0, 1)
+    return k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), ks, vs
+
+
+def _attention_ref(q, k, v, pos, scale, window):
+    """q [H, hd] at position pos over k, v [S, G, hd] in float64."""
+    H, hd = q.shape
+    G = k.shape[1]
+    lo = max(0, pos - window + 1) if window else 0
+    out = torch.empty(H, hd, dtype=torch.float64)
+    for h in range(H):
+        g = h // (H // G)
+        s = (k[lo:pos + 1, g].double() @ q[h].double()) * scale
+        out[h] = torch.softmax(s, 0) @ v[lo:pos + 1, g].double()
+    return out
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1.5e-2)])
+@pytest.mark.parametrize("H,G,hd,window", [(4, 4, 16, 0), (6, 2, 48, 0), (8, 1, 128, 0),
+                                           (3, 3, 80, 0), (4, 2, 64, 37), (2, 1, 256, 100)])
+def test_attention_over_pages(dtype, tol, H, G, hd, window):
+    """Prefill rows (many tokens of a sequence) and decode rows (its last token) in one
+    launch, sequences of unequal length on scattered pages, unused page tails poisoned."""
+    from gpt_fast_amd.ops import attention as A
+    lens = [1, 63, 64, 65, 200, 333]
+    k_pages, v_pages, table, ks, vs = _paged(lens, G, hd, dtype, seed=hd + H)
+    g = torch.Generator().manual_seed(5)
+    tok_seq, tok_pos = [], []
+    for b, S in enumerate(lens):
+        new = list(range(S)) if b % 2 == 0 else [S - 1]        # whole prompt / one token
+        tok_seq += [b] * len(new)
+        tok_pos += new
+    q = torch.randn(len(tok_seq), H, hd, generator=g).to(dtype)
+    scale = 1.0 / math.sqrt(hd)
+
+    class B:
+        pass
+    batch = B()
+    batch.tok_seq = torch.tensor(tok_seq, dtype=torch.int32, device=DEV)
+    batch.tok_pos = torch.tensor(tok_pos, dtype=torch.int32, device=DEV)
+    batch.n_tokens, batch.n_seqs = len(tok_seq), len(lens)
+    batch.max_q_len, batch.max_kv_len, batch.is_decode = max(lens), max(lens), False
+    starts = [0 if b % 2 == 0 else S - 1 for b, S in enumerate(lens)]
+    qs = [0]
+    for b, S in enumerate(lens):
+        qs.append(qs[-1] + (S if b % 2 == 0 else 1))
+    batch.q_start = torch.tensor(qs, dtype=torch.int32, device=DEV)
+    batch.start_pos = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    batch.host_q_start, batch.host_start_pos = qs, starts
+    out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, scale, window).cpu()
+    plain = K().attention_generic(q.to(DEV), k_pages, v_pages, batch.tok_seq, batch.tok_pos,
+                                  table, scale, window).cpu()
+    assert not torch.isnan(out).any()
+    for n in range(len(tok_seq)):
+        b, p = tok_seq[n], tok_pos[n]
+        ref = _attention_ref(q[n].float(), ks[b].float(), vs[b].float(), p, scale, window)
+        close(out[n], ref, tol)
+        close(plain[n], ref, tol)
+
+
+def test_attention_finds_one_far_key():
+    """One key among hundreds stands out (its score is scaled up): the output must be
+    that key's value, wherever in the cache it lies - first row, a page edge, the last."""
+    from gpt_fast_amd.ops import attention as A
+    H, G, hd, S = 4, 2, 64, 700
+    for dtype in (torch.float32, torch.bfloat16):
+        for target in (0, 63, 64, 511, 699):
+            k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=target)
+            q = torch.zeros(1, H, hd)
+            for h in range(H):
+                q[0, h] = ks[0][target, h // 2].float() * 40.0
+            q = q.to(dtype)
+
+            class B:
+                pass
+            batch = B()
+            batch.tok_seq = torch.zeros(1, dtype=torch.int32, device=DEV)
+            batch.tok_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
+            batch.n_tokens = batch.n_seqs = 1
+            batch.max_q_len, batch.max_kv_len, batch.is_decode = 1, S, True
+            batch.q_start = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+            batch.start_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
+            batch.host_q_start, batch.host_start_pos = [0, 1], [S - 1]
+            out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, 1.0, 0).cpu().float()
+            for h in range(H):
+                close(out[0, h], vs[0][target, h // 2].float(), 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layout", [0, 1])
+@pytest.mark.parametrize("H,G,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 2, 128, 128)])
+def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):
+    torch.manual_seed(6)
+    pos = [0, 1, 63, 64, 130, 4000]
+    N = len(pos)
+    qkv = torch.randn(N, (H + 2 * G) * hd).to(dtype)
+    freqs = 1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))
+    table = torch.tensor([[5, 3, 0, 1] + [2] * 60], dtype=torch.int32)
+    k_pages = torch.zeros(6, G, 64, hd).to(dtype)
+    v_pages = torch.zeros(6, G, 64, hd).to(dtype)
+    kp, vp = k_pages.to(DEV), v_pages.to(DEV)
+    q_out = K().rope_cache_write(
+        qkv.to(DEV), freqs.to(DEV), torch.zeros(N, dtype=torch.int32, device=DEV),
+        torch.tensor(pos, dtype=torch.int32, device=DEV), table.to(DEV), kp, vp, H, G, hd, rot,
+        layout).cpu().float()
+    x = qkv.float().reshape(N, H + 2 * G, hd)
+    ang = torch.tensor(pos, dtype=torch.float32)[:, None] * freqs[None, :]
+    c, s = torch.cos(ang.double())[:, None, :], torch.sin(ang.double())[:, None, :]
+    ref = x.double().clone()
+    qk = x[:, :H + G].double()
+    if layout == 0:
+        a, b = qk[..., 0:rot:2], qk[..., 1:rot:2]
+        ref[:, :H + G, 0:rot:2] = a * c - b * s
+        ref[:, :H + G, 1:rot:2] = b * c + a * s
+    else:
+        a, b = qk[..., :rot // 2], qk[..., rot // 2:rot]
+        ref[:, :H + G, :rot // 2] = a * c - b * s
+        ref[:, :H + G, rot // 2:rot] = b * c + a * s
+    tol = 2e-4 if dtype == torch.float32 else 1e-2      # float: cos/sin of angles up to 4000
+    close(q_out, ref[:, :H], tol)
+    kc, vc = kp.cpu().float(), vp.cpu().float()
+    for n, p in enumerate(pos):
+        page = int(table[0, p // 64])
+        close(kc[page, :, p % 64], ref[n, H:H + G], tol)
+        assert torch.equal(vc[page, :, p % 64], x[n, H + G:])
+    # rotary_dim 0 and no pages: q passes through, nothing is written
+    q2 = K().rope_cache_write(qkv.to(DEV), None, torch.zeros(N, dtype=torch.int32, device=DEV),
+                              torch.tensor(pos, dtype=torch.int32, device=DEV), table.to(DEV),
+                              None, None, H, G, hd, 0, 0).cpu()
+    assert torch.equal(q2.reshape(N, -1), qkv[:, :H * hd])
+
+
+def test_argmax_and_sampling():
+    from gpt_fast_amd.sampling import SamplingParams, logits_to_probs, sample
+    import plain_llama as plain
+    torch.manual_seed(7)
+    B, V = 5, 1000
+    logits = torch.randn(B, V, device=DEV) * 3
+    logits[2, 17] = logits[2, 400] = 50.0                       # tie: the lowest index wins
+    logits[3, 5] = float("nan")
+    keys = torch.arange(B, dtype=torch.int32, device=DEV)
+    got = K().argmax(logits).cpu()
+    assert got[2] == 17
+    clean = torch.nan_to_num(logits, nan=-1e30)
+    assert torch.equal(got.long(), clean.argmax(-1).cpu())
+    greedy = sample(logits, SamplingParams(temperature=0.0), keys, None)
+    assert torch.equal(greedy.cpu(), got)
+
+    logits = torch.randn(B, V, device=DEV) * 2
+    for T, k in ((0.8, 50), (1.0, None), (0.3, 1), (1.5, 2000), (0.7, 7)):
+        p = logits_to_probs(logits, T, k).cpu()
+        ref = plain.logits_to_probs(logits.cpu(), T, k)
+        assert torch.allclose(p, ref, rtol=1e-4, atol=1e-7), (T, k)
+        if k is not None and k < V:
+            assert ((p > 0).sum(-1) == k).all()
+    top1 = sample(logits, SamplingParams(temperature=0.9, top_k=1, seed=3), keys, None)
+    assert torch.equal(top1.cpu().long(), logits.argmax(-1).cpu())
+    # ties with the k-th value survive
+    tie = torch.zeros(1, 10, device=DEV)
+    tie[0, :3] = 2.0
+    tie[0, 3:6] = 1.0
+    assert int((logits_to_probs(tie, 1.0, 4) > 0).sum()) == 6
+
+    # frequencies follow the probabilities (chi-square, 3 degrees of freedom)
+    small = torch.log(torch.tensor([[0.5, 0.25, 0.15, 0.1]], device=DEV)).repeat(4000, 1)
+    rows = torch.arange(4000, dtype=torch.int32, device=DEV)
+    draws = sample(small, SamplingParams(temperature=1.0, seed=11), rows, None).cpu()
+    counts = torch.bincount(draws.long(), minlength=4).double()
+    expect = torch.tensor([0.5, 0.25, 0.15, 0.1]).double() * 4000
+    assert float(((counts - expect) ** 2 / expect).sum()) < 16.3      # p = 0.001
+
+    # a row's draw depends on (seed, key, position) only, not on its place in the batch
+    params = SamplingParams(temperature=1.0, top_k=100, seed=5)
+    pos = torch.tensor([4, 9, 2, 7, 7], dtype=torch.int32, device=DEV)
+    a = sample(logits, params, keys, pos, 1).cpu()
+    order = torch.tensor([3, 0, 4, 2, 1], device=DEV)
+    b = sample(logits[order].contiguous(), params, keys[order].contiguous(),
+               pos[order].contiguous(), 1).cpu()
+    assert torch.equal(b, a[order.cpu()])
+    c = sample(logits, SamplingParams(temperature=1.0, top_k=100, seed=6), keys, pos, 1).cpu()
+    assert not torch.equal(a, c)

@@ -54,9 +54,12 @@ class KVGroup:
         self.need = need
         self.entries = entries
         self.n_pages = n_pages
-        shape = (entries, n_pages, need.n_kv_heads, PAGE, need.head_dim)
-        self.k = torch.empty(shape, dtype=dtype, device=device)
-        self.v = torch.empty(shape, dtype=dtype, device=device)
+        # keys as rows [PAGE, head_dim]; values transposed [head_dim, PAGE]: the operand
+        # layouts of the matrix-core attention kernel
+        self.k = torch.empty((entries, n_pages, need.n_kv_heads, PAGE, need.head_dim),
+                             dtype=dtype, device=device)
+        self.v = torch.empty((entries, n_pages, need.n_kv_heads, need.head_dim, PAGE),
+                             dtype=dtype, device=device)
         self.pages = FreeList(n_pages, "cache page")
         self.held: Dict[int, List[int]] = {}      # slot -> page of each PAGE tokens, -1 = given back
 

@@ -83,4 +83,12 @@ __device__ __forceinline__ size_t page_row(int page, int kv_head, int offset, in
     return (((size_t)page * n_kv_heads + kv_head) * GFA_PAGE + offset) * (size_t)head_dim;
 }
 
+// Values are kept transposed: one layer's pool is [n_pages, n_kv_heads, head_dim, GFA_PAGE],
+// so that the keys of a page are contiguous for each element of the head.  The matrix-core
+// attention reads its value operand (8 consecutive keys per lane) straight from this layout.
+__device__ __forceinline__ size_t value_elem(int page, int kv_head, int d, int offset,
+                                             int n_kv_heads, int head_dim) {
+    return (((size_t)page * n_kv_heads + kv_head) * head_dim + d) * GFA_PAGE + offset;
+}
+
 #define GFA_LAUNCH_RESULT() ((int)hipGetLastError())

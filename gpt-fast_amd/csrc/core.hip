@@ -135,7 +135,8 @@ extern "C" int gfa_gemm_f32(const float* a, const float* w, float* out, int M, i
 // Pair i of a head is (2i, 2i+1) if layout == 0 (model.py:281-293) or (i, i + rot/2) if
 // layout == 1; it is rotated by angle = float(position) * freqs[i], cos and sin in float.
 // Elements beyond `rot` pass through.  q goes to q_out [N, H, hd]; k and v of token n go
-// to page table[seq(n)][pos / PAGE], offset pos % PAGE (model.py:91-100, 206-207).
+// to page table[seq(n)][pos / PAGE], offset pos % PAGE (model.py:91-100, 206-207); keys as
+// rows [offset, hd], values transposed [hd, offset] (see common.h).
 template <typename T>
 __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                   T* __restrict__ k_pages, T* __restrict__ v_pages,
@@ -150,9 +151,10 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
     const int half = hd / 2;          // pairs per head when every element had a partner
     const int rot_pairs = rot / 2;
     size_t kv_base = 0;
+    int v_page = 0;
     if (k_pages) {
-        const int page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
-        kv_base = page_row(page, 0, pos % GFA_PAGE, Hkv, hd);
+        v_page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+        kv_base = page_row(v_page, 0, pos % GFA_PAGE, Hkv, hd);
     }
     // q and k heads: one thread per (head, pair-or-passthrough slot)
     const int n_rot_heads = H + Hkv;
@@ -185,7 +187,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
         const T* vsrc = row + (size_t)(H + Hkv) * hd;
         for (int e = threadIdx.x; e < Hkv * hd; e += blockDim.x) {
             const int g = e / hd, d = e % hd;
-            v_pages[kv_base + (size_t)g * GFA_PAGE * hd + d] = vsrc[e];
+            v_pages[value_elem(v_page, g, d, pos % GFA_PAGE, Hkv, hd)] = vsrc[e];
         }
     }
 }
@@ -261,9 +263,9 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
                 float a = acc[i] * alpha;
                 for (int jj = 0; jj < count; ++jj) {
                     const int key = base + jj;
-                    const T* vr = v_pages + page_row(pages[key / GFA_PAGE], g, key % GFA_PAGE,
-                                                     Hkv, hd);
-                    a = fmaf(sc[jj], load_as_float(vr + d), a);
+                    const T* vr = v_pages + value_elem(pages[key / GFA_PAGE], g, d,
+                                                       key % GFA_PAGE, Hkv, hd);
+                    a = fmaf(sc[jj], load_as_float(vr), a);
                 }
                 acc[i] = a;
             }

@@ -1,6 +1,62 @@
-"""Python faces of the bfloat16 attention kernels (csrc/attention_bf16.hip)."""
+"""Python face of the matrix-core attention kernel (csrc/attention_bf16.hip)."""
+import ctypes
+
+import torch
+
+from .library import KernelError, check, library, ptr, require_contiguous, require_device, stream_handle
+
+_i = ctypes.c_int
+_f = ctypes.c_float
+
+TARGET_WAVES = 512         # single-token steps split the context until this many waves run
+MIN_KEYS_PER_SPLIT = 128
+MAX_SPLITS = 16
+
+
+def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int):
+    """(row tiles per wave, waves per sequence and kv head, context splits) for a step."""
+    R = H // G
+    if max_q_len == 1:
+        rt = 1
+        tiles = (R + 15) // 16
+        waves = n_seqs * G * tiles
+        splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS,
+                     max(1, table_width * 64 // MIN_KEYS_PER_SPLIT))
+        return rt, tiles, max(splits, 1)
+    rt = 4 if hd <= 128 else 2
+    rows = max_q_len * R
+    if rows <= 16:
+        rt = 1
+    elif rows <= 32:
+        rt = min(rt, 2)
+    return rt, (rows + 16 * rt - 1) // (16 * rt), 1
 
 
 def attention(q, k_pages, v_pages, batch, table, scale, window):
-    """The fast kernel's result, or None if no fast kernel takes this shape."""
-    return None
+    """The kernel's result [N, H, hd], or None if it does not take this shape (head sizes
+    that are no multiple of 16 or exceed 256 go to the plain kernel)."""
+    n, H, hd = q.shape
+    G = k_pages.shape[1]
+    if hd % 16 or hd > 256 or H % G:
+        return None
+    require_device(q, k_pages, v_pages, table, batch.q_start, batch.start_pos)
+    require_contiguous(q=q, k_pages=k_pages, v_pages=v_pages, table=table)
+    if q.dtype != torch.bfloat16 or k_pages.dtype != torch.bfloat16 or v_pages.dtype != torch.bfloat16:
+        raise KernelError("attention_bf16: bfloat16 tensors only")
+    if tuple(k_pages.shape[1:]) != (G, 64, hd) or tuple(v_pages.shape[1:]) != (G, hd, 64):
+        raise KernelError(f"attention_bf16: pages are {tuple(k_pages.shape)} / {tuple(v_pages.shape)}")
+    if batch.q_start.numel() != batch.n_seqs + 1 or batch.start_pos.numel() != batch.n_seqs \
+            or table.shape[0] != batch.n_seqs or table.dtype != torch.int32:
+        raise KernelError("attention_bf16: the batch description does not fit its sequences")
+    rt, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
+    out = torch.empty_like(q)
+    ws_o = ws_ml = None
+    if splits > 1:
+        ws_o = torch.empty((splits, n * H, hd), dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty((splits, n * H, 2), dtype=torch.float32, device=q.device)
+    check(library("attention_bf16").gfa_attention_bf16(
+        ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos), ptr(table),
+        _i(table.shape[1]), ptr(out), ptr(ws_o), ptr(ws_ml), _i(n), _i(batch.n_seqs), _i(H), _i(G),
+        _i(hd), _f(scale), _i(window), _i(rt), _i(tiles), _i(splits), stream_handle()),
+        "attention_bf16")
+    return out

@@ -8,6 +8,15 @@ from .library import KernelError, check, library, ptr, require_contiguous, requi
 
 _i = ctypes.c_int
 MAX_ROWS = 64
+# rows of x up to which the dot-product kernel is used; above, the matrix-core kernel
+DOT_MAX_ROWS = 1
+
+
+def _entry(M: int, K: int):
+    lib = library("gemm_bf16")
+    if M > DOT_MAX_ROWS and K % 8 == 0:
+        return lib.gfa_skinny_mfma_bf16
+    return lib.gfa_skinny_bf16
 
 
 def _check_operands(x, w, what):
@@ -44,8 +53,8 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         elif out.shape != (M, N) or out.dtype != out_dtype or not out.is_contiguous():
             raise KernelError("skinny: out has the wrong shape or dtype")
         mode = 0 if out_dtype == torch.bfloat16 else 1
-    check(library("gemm_bf16").gfa_skinny_bf16(ptr(x), ptr(w), ptr(out), _i(M), _i(N), _i(K),
-                                               _i(N), _i(mode), _i(0), stream_handle()), "skinny")
+    check(_entry(M, K)(ptr(x), ptr(w), ptr(out), _i(M), _i(N), _i(K), _i(N), _i(mode), _i(0),
+                       stream_handle()), "skinny")
     return out
 
 
@@ -60,9 +69,8 @@ def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor]
         out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
     elif out.shape != (M, I) or out.dtype != torch.bfloat16 or not out.is_contiguous():
         raise KernelError("skinny_gated: out has the wrong shape or dtype")
-    check(library("gemm_bf16").gfa_skinny_bf16(ptr(x), ptr(w13), ptr(out), _i(M), _i(I), _i(K),
-                                               _i(I), _i(3), _i(I), stream_handle()),
-          "skinny_gated")
+    check(_entry(M, K)(ptr(x), ptr(w13), ptr(out), _i(M), _i(I), _i(K), _i(I), _i(3), _i(I),
+                       stream_handle()), "skinny_gated")
     return out
 
 

@@ -119,11 +119,12 @@ def gemm_bf16_naive(a: torch.Tensor, w: torch.Tensor):
 
 # ----------------------------------------------------------------------------- rope + cache
 def _check_pages(k_pages, v_pages, n_kv_heads, head_dim, dtype):
-    for name, p in (("k_pages", k_pages), ("v_pages", v_pages)):
+    for name, p, tail in (("k_pages", k_pages, (n_kv_heads, PAGE, head_dim)),
+                          ("v_pages", v_pages, (n_kv_heads, head_dim, PAGE))):
         if p is None:
             continue
-        if p.dim() != 4 or p.shape[1:] != (n_kv_heads, PAGE, head_dim):
-            raise KernelError(f"{name} must be [n_pages, {n_kv_heads}, {PAGE}, {head_dim}], "
+        if p.dim() != 4 or tuple(p.shape[1:]) != tail:
+            raise KernelError(f"{name} must be [n_pages, {tail[0]}, {tail[1]}, {tail[2]}], "
                               f"is {tuple(p.shape)}")
         if p.dtype != dtype or not p.is_contiguous():
             raise KernelError(f"{name} must be contiguous {dtype}")

@@ -55,6 +55,7 @@ def test_groups_by_need():
     assert c.entries[0].group_id == c.entries[2].group_id != c.entries[1].group_id
     assert (c.entries[0].index, c.entries[2].index) == (0, 1)
     assert c.groups[c.entries[0].group_id].k.shape == (2, 6, 2, 64, 8)
+    assert c.groups[c.entries[0].group_id].v.shape == (2, 6, 2, 8, 64)
     assert c.entries[3].state.shape == (4, 3)
     # a borrowed entry reads the lender's storage and does not write
     b = Cache([KVNeed(1, 8), KVNeed(1, 8)], [None, 0], max_tokens=64, max_sequences=1,

@@ -106,7 +106,7 @@ def _paged(S_list, G, hd, dtype, seed):
     n_pages = sum((s + 63) // 64 for s in S_list) + 3
     perm = torch.randperm(n_pages, generator=g).tolist()
     k_pages = torch.full((n_pages, G, 64, hd), float("nan")).to(dtype)      # poison: never read
-    v_pages = torch.full((n_pages, G, 64, hd), float("nan")).to(dtype)
+    v_pages = torch.full((n_pages, G, hd, 64), float("nan")).to(dtype)     # values transposed
     width = max((s + 63) // 64 for s in S_list)
     table = torch.full((len(S_list), width), -1, dtype=torch.int32)
     ks, vs = [], []
@@ -120,7 +120,7 @@ def _paged(S_list, G, hd, dtype, seed):
             table[b, i] = p
             n = min(64, S - 64 * i)
             k_pages[p, :, :n] = k[64 * i:64 * i + n].transpose(0, 1)
-            v_pages[p, :, :n] = v[64 * i:64 * i + n].transpose(0, 1)
+            v_pages[p, :, :, :n] = v[64 * i:64 * i + n].permute(1, 2, 0)
     return k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), ks, vs
 
 
@@ -219,7 +219,7 @@ def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):
     freqs = 1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))
     table = torch.tensor([[5, 3, 0, 1] + [2] * 60], dtype=torch.int32)
     k_pages = torch.zeros(6, G, 64, hd).to(dtype)
-    v_pages = torch.zeros(6, G, 64, hd).to(dtype)
+    v_pages = torch.zeros(6, G, hd, 64).to(dtype)
     kp, vp = k_pages.to(DEV), v_pages.to(DEV)
     q_out = K().rope_cache_write(
         qkv.to(DEV), freqs.to(DEV), torch.zeros(N, dtype=torch.int32, device=DEV),
@@ -244,7 +244,7 @@ def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):
     for n, p in enumerate(pos):
         page = int(table[0, p // 64])
         close(kc[page, :, p % 64], ref[n, H:H + G], tol)
-        assert torch.equal(vc[page, :, p % 64], x[n, H + G:])
+        assert torch.equal(vc[page, :, :, p % 64], x[n, H + G:])
     # rotary_dim 0 and no pages: q passes through, nothing is written
     q2 = K().rope_cache_write(qkv.to(DEV), None, torch.zeros(N, dtype=torch.int32, device=DEV),
                               torch.tensor(pos, dtype=torch.int32, device=DEV), table.to(DEV),

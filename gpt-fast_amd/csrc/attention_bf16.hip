@@ -35,22 +35,24 @@ union Frag {
 
 #define LOG2E 1.4426950408889634f
 
-template <int DS, int RT>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+template <int DS, int RT, bool PREFETCH>
+__global__ __launch_bounds__(256) void attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
         bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
         int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows) {
     constexpr int DT = DS * 2;
-    const int lane = threadIdx.x, li = lane & 15, lg = lane >> 4;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
     const int g = blockIdx.y;
     const int seq = blockIdx.z / n_splits, split = blockIdx.z - seq * n_splits;
     const int R = H / Hkv;
     const int q0 = q_start[seq];
     const int rows_total = (q_start[seq + 1] - q0) * R;
     const int row0 = blockIdx.x * 16 * RT;
-    if (row0 >= rows_total) return;
+    if (row0 >= rows_total) return;                      // the whole workgroup leaves
     const int spos = start_pos[seq];
     const int* pages = table + (size_t)seq * table_stride;
 
@@ -88,31 +90,20 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int kb = kb_begin; kb < kb_end; ++kb) {
+    // keys: tile kt, row kt * 16 + li of the block, dims ds * 32 + lg * 8 .. +7
+    // values: dims dt * 16 + li, keys (tile 0 | tile 1) 4 lg .. +3 of the block
+    auto load_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
         const int page = pages[kb >> 1];
         const int in_page = (kb & 1) * 32;
         const bf16_t* kbase = k_pages + page_row(page, g, in_page, Hkv, hd);
-        floatx4_t s[RT][2];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            Frag kf[DS];
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) {
                 const int d = ds * 32 + lg * 8;
-                kf[ds].u = (d < hd) ? *(const uint4*)(kbase + (size_t)(kt * 16 + li) * hd + d)
-                                    : make_uint4(0, 0, 0, 0);
+                kf[kt][ds].u = (d < hd) ? *(const uint4*)(kbase + (size_t)(kt * 16 + li) * hd + d)
+                                        : make_uint4(0, 0, 0, 0);
             }
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                s[rt][kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ds = 0; ds < DS; ++ds)
-                    s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ds].v, qf[rt][ds].v, s[rt][kt], 0, 0, 0);
-            }
-        }
-        // values: dims dt * 16 + li, keys (tile 0 | tile 1) 4 lg .. +3 of this block
-        Frag vf[DT];
-        const int key0 = kb * 32 + lg * 4;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const int d = dt * 16 + li;
@@ -124,6 +115,19 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
                 vf[dt].u = make_uint4(0, 0, 0, 0);
             }
         }
+    };
+    auto compute_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
+        const int key0 = kb * 32 + lg * 4;
+        floatx4_t s[RT][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                s[rt][kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < DS; ++ds)
+                    s[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][ds].v, qf[rt][ds].v, s[rt][kt], 0, 0, 0);
+            }
         if (kb * 32 + 31 > pmax) {          // slots beyond the newest key hold no data yet
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -165,15 +169,74 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
                 }
             }
         }
+    };
+
+    // the waves of a workgroup take the blocks of their share in turn
+    int kb = kb_begin + wave;
+    if (PREFETCH) {
+        Frag kfa[2][DS], vfa[DT], kfb[2][DS], vfb[DT];
+        if (kb < kb_end) load_block(kb, kfa, vfa);
+        for (; kb < kb_end; kb += 2 * nw) {
+            const bool more = kb + nw < kb_end;
+            if (more) load_block(kb + nw, kfb, vfb);
+            compute_block(kb, kfa, vfa);
+            if (more) {
+                if (kb + 2 * nw < kb_end) load_block(kb + 2 * nw, kfa, vfa);
+                compute_block(kb + nw, kfb, vfb);
+            }
+        }
+    } else {
+        Frag kfa[2][DS], vfa[DT];
+        for (; kb < kb_end; kb += nw) {
+            load_block(kb, kfa, vfa);
+            compute_block(kb, kfa, vfa);
+        }
+    }
+
+    float lt[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        lt[rt] = l[rt] + __shfl_xor(l[rt], 16, 64);
+        lt[rt] += __shfl_xor(lt[rt], 32, 64);
+    }
+    if (nw > 1) {                 // the waves' partial results meet in LDS, added in wave order
+        float* sm_ml = (float*)smem;                                  // [nw][RT][16][2]
+        floatx4_t* sm_o = (floatx4_t*)(smem + (size_t)nw * RT * 16 * 2 * sizeof(float));
+        if (wave > 0) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                if (lg == 0) {
+                    sm_ml[((wave * RT + rt) * 16 + li) * 2] = m[rt];
+                    sm_ml[((wave * RT + rt) * 16 + li) * 2 + 1] = lt[rt];
+                }
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) sm_o[((wave * RT + rt) * DT + dt) * 64 + lane] = o[rt][dt];
+            }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 1; w < nw; ++w)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const float mw = sm_ml[((w * RT + rt) * 16 + li) * 2];
+                if (mw == -INFINITY) continue;
+                const float lw = sm_ml[((w * RT + rt) * 16 + li) * 2 + 1];
+                const float m_new = fmaxf(m[rt], mw);
+                const float a = __builtin_amdgcn_exp2f(m[rt] - m_new);     // 0 if this wave saw no key
+                const float b = __builtin_amdgcn_exp2f(mw - m_new);
+                lt[rt] = lt[rt] * a + lw * b;
+                m[rt] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    o[rt][dt] = o[rt][dt] * a + sm_o[((w * RT + rt) * DT + dt) * 64 + lane] * b;
+            }
     }
 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        float lt = l[rt] + __shfl_xor(l[rt], 16, 64);
-        lt += __shfl_xor(lt, 32, 64);
         if (rpos[rt] < 0) continue;
         if (n_splits == 1) {
-            const float inv = 1.f / lt;
+            const float inv = 1.f / lt[rt];
             bf16_t* orow_p = out + orow[rt] * hd;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
@@ -195,7 +258,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
             }
             if (lg == 0) {
                 ws_ml[prow * 2] = m[rt];
-                ws_ml[prow * 2 + 1] = lt;
+                ws_ml[prow * 2 + 1] = lt[rt];
             }
         }
     }
@@ -223,33 +286,36 @@ __global__ void attention_combine_kernel(const float* __restrict__ ws_o,
 }
 
 template <int DS>
-static void launch_attention(int rt, dim3 grid, hipStream_t stream, const bf16_t* q,
+static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, const bf16_t* q,
                              const bf16_t* k, const bf16_t* v, const int* q_start,
                              const int* start_pos, const int* table, int table_stride, bf16_t* out,
                              float* ws_o, float* ws_ml, int H, int Hkv, int hd, float sl2, int window,
                              int n_splits, int total_rows) {
+    const size_t shmem = nw > 1 ? (size_t)nw * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
     if (rt == 1)
-        attention_mfma_kernel<DS, 1><<<grid, 64, 0, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     else if (rt == 2)
-        attention_mfma_kernel<DS, 2><<<grid, 64, 0, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
-    else
-        attention_mfma_kernel<DS, 4><<<grid, 64, 0, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+    else if (DS <= 4)
+        attention_mfma_kernel<(DS <= 4 ? DS : 4), 4, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
 }
 
 // q, out [n_tokens, H, hd]; the sequences' token runs are given by q_start [n_seqs + 1] and
 // their first positions by start_pos [n_seqs].  rt (1, 2 or 4) 16-row tiles per wave;
+// n_waves (1..4) waves per workgroup share the key blocks of their rows;
 // max_tiles = most waves any sequence needs per kv head.  With n_splits > 1, ws_o
 // [n_splits, n_tokens * H, hd] and ws_ml [n_splits, n_tokens * H, 2] hold the partials.
 extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void* v_pages,
                                   const int* q_start, const int* start_pos, const int* table,
                                   int table_stride, void* out, float* ws_o, float* ws_ml,
                                   int n_tokens, int n_seqs, int H, int Hkv, int hd, float scale,
-                                  int window, int rt, int max_tiles, int n_splits,
+                                  int window, int rt, int n_waves, int max_tiles, int n_splits,
                                   hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || max_tiles < 1 ||
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
-        (n_splits > 1 && (!ws_o || !ws_ml)))
+        (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > 4 ||
+        (size_t)n_waves * rt * (128 + (hd <= 64 ? 2 : hd <= 128 ? 4 : 8) * 2 * 1024) > 65536)
         return (int)hipErrorInvalidValue;
     const dim3 grid(max_tiles, Hkv, n_seqs * n_splits);
     const float sl2 = scale * LOG2E;
@@ -258,11 +324,11 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     const bf16_t* kp = (const bf16_t*)k_pages;
     const bf16_t* vp = (const bf16_t*)v_pages;
     if (hd <= 64)
-        launch_attention<2>(rt, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<2>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     else if (hd <= 128)
-        launch_attention<4>(rt, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<4>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     else
-        launch_attention<8>(rt, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     if (n_splits > 1)
         attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows);
     return GFA_LAUNCH_RESULT();

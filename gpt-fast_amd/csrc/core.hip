@@ -52,9 +52,62 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int d = threadIdx.x; d < dim; d += blockDim.x) store_from_float(o + d, xr[d] * rs * w[d]);
 }
 
+// The same for rows of up to 1024 * VPT elements (a multiple of 4): the row is read once
+// with 16-byte loads, kept in registers between the sum and the scaling.
+template <typename T, int VPT>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
+        const float* __restrict__ x, const float* __restrict__ w, const int* __restrict__ rows,
+        T* __restrict__ out, int dim, float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    const float4* xr = (const float4*)(x + (size_t)r * dim);
+    const float4* w4 = (const float4*)w;
+    const int n4 = dim >> 2;
+    float4 v[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * 256;
+        v[j] = idx < n4 ? xr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss = fmaf(v[j].x, v[j].x, ss);
+        ss = fmaf(v[j].y, v[j].y, ss);
+        ss = fmaf(v[j].z, v[j].z, ss);
+        ss = fmaf(v[j].w, v[j].w, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float rs = rsqrtf(ss / (float)dim + eps);
+    T* o = out + (size_t)i * dim;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * 256;
+        if (idx < n4) {
+            const float4 g = w4[idx];
+            store_from_float(o + 4 * idx + 0, v[j].x * rs * g.x);
+            store_from_float(o + 4 * idx + 1, v[j].y * rs * g.y);
+            store_from_float(o + 4 * idx + 2, v[j].z * rs * g.z);
+            store_from_float(o + 4 * idx + 3, v[j].w * rs * g.w);
+        }
+    }
+}
+
+template <typename T>
+static bool launch_rmsnorm_vec(const float* x, const float* w, const int* rows, T* out, int n_rows,
+                               int dim, float eps, hipStream_t stream) {
+    if (dim % 4 != 0 || dim > 8192) return false;
+    if (dim <= 1024) rmsnorm_vec_kernel<T, 1><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    else if (dim <= 2048) rmsnorm_vec_kernel<T, 2><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    else if (dim <= 4096) rmsnorm_vec_kernel<T, 4><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    else rmsnorm_vec_kernel<T, 8><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    return true;
+}
+
 extern "C" int gfa_rmsnorm(const float* x, const float* w, const int* rows, void* out,
                            int out_bf16, int n_rows, int dim, float eps, hipStream_t stream) {
     if (n_rows <= 0) return 0;
+    if (out_bf16 ? launch_rmsnorm_vec<bf16_t>(x, w, rows, (bf16_t*)out, n_rows, dim, eps, stream)
+                 : launch_rmsnorm_vec<float>(x, w, rows, (float*)out, n_rows, dim, eps, stream))
+        return GFA_LAUNCH_RESULT();
     if (out_bf16)
         rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, w, rows, (bf16_t*)out, dim, eps);
     else
@@ -156,6 +209,11 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
         v_page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
         kv_base = page_row(v_page, 0, pos % GFA_PAGE, Hkv, hd);
     }
+    // cos and sin of this token's angles, once for all heads
+    extern __shared__ float cs[];                  // [rot_pairs][2]
+    for (int i = threadIdx.x; i < rot_pairs; i += blockDim.x)
+        sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
+    __syncthreads();
     // q and k heads: one thread per (head, pair-or-passthrough slot)
     const int n_rot_heads = H + Hkv;
     for (int e = threadIdx.x; e < n_rot_heads * half; e += blockDim.x) {
@@ -172,8 +230,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
             const int ia = layout == 0 ? 2 * i : i;
             const int ib = layout == 0 ? 2 * i + 1 : i + rot_pairs;
             const float a = load_as_float(src + ia), b = load_as_float(src + ib);
-            float s, c;
-            sincosf((float)pos * freqs[i], &s, &c);
+            const float c = cs[2 * i], s = cs[2 * i + 1];
             store_from_float(dst + ia, a * c - b * s);
             store_from_float(dst + ib, b * c + a * s);
         } else {
@@ -199,11 +256,11 @@ extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages,
                                     hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (is_bf16)
-        rope_cache_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(
+        rope_cache_kernel<bf16_t><<<n_tokens, 256, (size_t)rot * sizeof(float), stream>>>(
             (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs,
             tok_seq, tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     else
-        rope_cache_kernel<float><<<n_tokens, 256, 0, stream>>>(
+        rope_cache_kernel<float><<<n_tokens, 256, (size_t)rot * sizeof(float), stream>>>(
             (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, freqs, tok_seq,
             tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     return GFA_LAUNCH_RESULT();

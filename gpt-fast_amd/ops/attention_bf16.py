@@ -8,28 +8,33 @@ from .library import KernelError, check, library, ptr, require_contiguous, requi
 _i = ctypes.c_int
 _f = ctypes.c_float
 
-TARGET_WAVES = 512         # single-token steps split the context until this many waves run
+TARGET_WAVES = 1024        # single-token steps split the context until this many waves run
 MIN_KEYS_PER_SPLIT = 128
 MAX_SPLITS = 16
 
 
+PREFILL_ROW_TILES = 4      # 16-row tiles per wave for prompts
+
+
 def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int):
-    """(row tiles per wave, waves per sequence and kv head, context splits) for a step."""
+    """(row tiles per wave, waves per workgroup, workgroups per sequence and kv head,
+    context splits) for a step."""
     R = H // G
     if max_q_len == 1:
         rt = 1
+        nw = 4 if hd <= 128 else 2
         tiles = (R + 15) // 16
-        waves = n_seqs * G * tiles
+        waves = n_seqs * G * tiles * nw
         splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS,
-                     max(1, table_width * 64 // MIN_KEYS_PER_SPLIT))
-        return rt, tiles, max(splits, 1)
-    rt = 4 if hd <= 128 else 2
+                     max(1, table_width * 64 // (MIN_KEYS_PER_SPLIT * nw)))
+        return rt, nw, tiles, max(splits, 1)
+    rt = PREFILL_ROW_TILES if hd <= 128 else min(PREFILL_ROW_TILES, 2)
     rows = max_q_len * R
     if rows <= 16:
         rt = 1
     elif rows <= 32:
         rt = min(rt, 2)
-    return rt, (rows + 16 * rt - 1) // (16 * rt), 1
+    return rt, 1, (rows + 16 * rt - 1) // (16 * rt), 1
 
 
 def attention(q, k_pages, v_pages, batch, table, scale, window):
@@ -48,7 +53,7 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
     if batch.q_start.numel() != batch.n_seqs + 1 or batch.start_pos.numel() != batch.n_seqs \
             or table.shape[0] != batch.n_seqs or table.dtype != torch.int32:
         raise KernelError("attention_bf16: the batch description does not fit its sequences")
-    rt, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
+    rt, nw, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
     out = torch.empty_like(q)
     ws_o = ws_ml = None
     if splits > 1:
@@ -57,6 +62,6 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
     check(library("attention_bf16").gfa_attention_bf16(
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos), ptr(table),
         _i(table.shape[1]), ptr(out), ptr(ws_o), ptr(ws_ml), _i(n), _i(batch.n_seqs), _i(H), _i(G),
-        _i(hd), _f(scale), _i(window), _i(rt), _i(tiles), _i(splits), stream_handle()),
+        _i(hd), _f(scale), _i(window), _i(rt), _i(nw), _i(tiles), _i(splits), stream_handle()),
         "attention_bf16")
     return out

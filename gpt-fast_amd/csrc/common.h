@@ -20,12 +20,10 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even; NaN stays NaN (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    const __bf16 b = (__bf16)f;
+    return __builtin_bit_cast(bf16_t, b);
 }
 
 template <typename T> __device__ __forceinline__ float load_as_float(const T* p);

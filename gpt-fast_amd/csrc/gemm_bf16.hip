@@ -30,6 +30,7 @@ __device__ __forceinline__ float silu(float a) { return a / (1.f + expf(-a)); }
 
 template <int MODE>
 __device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, float v, float gate_v) {
+    if (MODE == 4) return;                     // the rotary epilogue stores by itself
     if (MODE == 0) {
         ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(v);
     } else if (MODE == 1) {
@@ -221,10 +222,30 @@ union Frag8 {
     bf16x8_t v;
 };
 
-template <int CT, int MODE>
+// What the fused variants need beside the product itself.
+struct SkinnyExtra {
+    // NORM: x is the float residual stream; the product takes x * norm_w rounded to
+    // bfloat16 and is scaled by rsqrt(mean(x^2) + eps) at the end (model.py:236-241)
+    const float* x_f32;
+    const float* norm_w;
+    float eps;
+    // MODE 4: the columns are q heads, k heads, v heads (model.py:195-199); q and k pairs
+    // (2i, 2i+1) are rotated by tok_pos * freqs[i] (model.py:281-293), q goes to q_out
+    // [M, H, hd], k and v into the pages (model.py:91-100) unless k_pages is null
+    bf16_t* q_out;
+    bf16_t* k_pages;
+    bf16_t* v_pages;
+    const float* freqs;
+    const int* tok_seq;
+    const int* tok_pos;
+    const int* table;
+    int table_stride, H, Hkv, hd, rot;
+};
+
+template <int CT, int MODE, bool NORM>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
-        int N, int K, int ldo, int gate_rows) {
+        int N, int K, int ldo, int gate_rows, SkinnyExtra ex) {
     constexpr int RT = (MODE == 3) ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
@@ -236,10 +257,13 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     const int t_begin = (int)((long)wave * T / NW), t_end = (int)((long)(wave + 1) * T / NW);
 
     floatx4_t acc[RT][CT];
+    float ssq[CT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int ct = 0; ct < CT; ++ct) {
+        ssq[ct] = 0.f;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     const bf16_t* wsrc[RT][4];
 #pragma unroll
@@ -250,8 +274,9 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             if (n >= N) n = N - 1;                       // clamped rows are computed, not stored
             wsrc[rt][j] = w + (size_t)(n + rt * gate_rows) * K + lchunk * 8;
         }
-    uint4 regs[RT][4];
-    auto load_piece = [&](int t) {
+    // two register sets: while piece t is multiplied, pieces t + 1 and t + 2 are in flight
+    uint4 regs_a[RT][4], regs_b[RT][4];
+    auto load_piece = [&](int t, uint4 (&regs)[RT][4]) {
         const int k = t * SM_SUBK + lchunk * 8;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
@@ -260,23 +285,61 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                 regs[rt][j] = (k < K) ? *(const uint4*)(wsrc[rt][j] + t * SM_SUBK)
                                       : make_uint4(0, 0, 0, 0);
     };
-    if (t_begin < t_end) load_piece(t_begin);
-    for (int t = t_begin; t < t_end; ++t) {
+    auto stage_piece = [&](uint4 (&regs)[RT][4]) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *(uint4*)(stage + rt * SM_TILE + (lrow + 4 * j) * SM_PITCH + lchunk * 16) = regs[rt][j];
-        if (t + 1 < t_end) load_piece(t + 1);
+    };
+    // The x fragments of a piece are requested before the prefetch of later pieces of W:
+    // loads return in order, so waiting for x must not mean waiting for the prefetch.
+    constexpr int XS = SM_SUBK / 32;
+    uint4 xraw[XS][CT];                                  // bfloat16 x, or converted below
+    float4 xf0[NORM ? XS : 1], xf1[NORM ? XS : 1], xg0[NORM ? XS : 1], xg1[NORM ? XS : 1];
+    auto load_x = [&](int t) {
 #pragma unroll
-        for (int s = 0; s < SM_SUBK / 32; ++s) {
+        for (int s = 0; s < XS; ++s) {
             const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
-            Frag8 b[CT];
+            if (NORM) {                                  // CT == 1
+                const bool ok = fi < M && kk < K;
+                const float* xr = ex.x_f32 + (size_t)(ok ? fi : 0) * K + (ok ? kk : 0);
+                const float* gr = ex.norm_w + (ok ? kk : 0);
+                xf0[s] = *(const float4*)xr;
+                xf1[s] = *(const float4*)(xr + 4);
+                xg0[s] = *(const float4*)gr;
+                xg1[s] = *(const float4*)(gr + 4);
+            } else {
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                const int m = ct * 16 + fi;
-                b[ct].u = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
-                                            : make_uint4(0, 0, 0, 0);
+                for (int ct = 0; ct < CT; ++ct) {
+                    const int m = ct * 16 + fi;
+                    xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
+                                                    : make_uint4(0, 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto multiply_piece = [&](int t) {
+#pragma unroll
+        for (int s = 0; s < XS; ++s) {
+            Frag8 b[CT];
+            if (NORM) {
+                const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
+                if (fi < M && kk < K) {
+                    const float4 a0 = xf0[s], a1 = xf1[s], g0 = xg0[s], g1 = xg1[s];
+                    ssq[0] += a0.x * a0.x + a0.y * a0.y + a0.z * a0.z + a0.w * a0.w +
+                              a1.x * a1.x + a1.y * a1.y + a1.z * a1.z + a1.w * a1.w;
+                    bf16_t* e = (bf16_t*)&b[0].u;
+                    e[0] = float_to_bf16(a0.x * g0.x); e[1] = float_to_bf16(a0.y * g0.y);
+                    e[2] = float_to_bf16(a0.z * g0.z); e[3] = float_to_bf16(a0.w * g0.w);
+                    e[4] = float_to_bf16(a1.x * g1.x); e[5] = float_to_bf16(a1.y * g1.y);
+                    e[6] = float_to_bf16(a1.z * g1.z); e[7] = float_to_bf16(a1.w * g1.w);
+                } else {
+                    b[0].u = make_uint4(0, 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s][ct];
             }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -287,37 +350,114 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                     acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[ct].v, acc[rt][ct], 0, 0, 0);
             }
         }
+    };
+    if (t_begin < t_end) load_piece(t_begin, regs_a);
+    if (t_begin + 1 < t_end) load_piece(t_begin + 1, regs_b);
+    for (int t = t_begin; t < t_end; t += 2) {
+        load_x(t);
+        stage_piece(regs_a);
+        if (t + 2 < t_end) load_piece(t + 2, regs_a);
+        multiply_piece(t);
+        if (t + 1 < t_end) {
+            load_x(t + 1);
+            stage_piece(regs_b);
+            if (t + 3 < t_end) load_piece(t + 3, regs_b);
+            multiply_piece(t + 1);
+        }
+    }
+    if (NORM) {                                          // this wave's share of sum x^2 of row fi
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            ssq[ct] += __shfl_xor(ssq[ct], 16, GFA_WAVE);
+            ssq[ct] += __shfl_xor(ssq[ct], 32, GFA_WAVE);
+        }
     }
     if (NW > 1) {
         __syncthreads();                                 // staging is done; reuse it for the sums
         floatx4_t* red = (floatx4_t*)smem;
+        float* red_s = (float*)(smem + (size_t)NW * RT * CT * 64 * sizeof(floatx4_t));
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) red[((wave * RT + rt) * CT + ct) * 64 + lane] = acc[rt][ct];
+        if (NORM && fg == 0) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) red_s[(wave * CT + ct) * 16 + fi] = ssq[ct];
+        }
         __syncthreads();
         if (wave != 0) return;
-        for (int wv = 1; wv < NW; ++wv)
+        for (int wv = 1; wv < NW; ++wv) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += red[((wv * RT + rt) * CT + ct) * 64 + lane];
+            if (NORM) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) ssq[ct] += red_s[(wv * CT + ct) * 16 + fi];
+            }
+        }
     }
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = ct * 16 + fi;
         if (m >= M) continue;
+        if (NORM) {
+            const float rs = rsqrtf(ssq[ct] / (float)K + ex.eps);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + fg * 4 + j;
-            if (n < N) skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
+            for (int rt = 0; rt < RT; ++rt) acc[rt][ct] *= rs;
+        }
+        if (MODE == 4) {
+            // columns n0 + 4 fg .. +3 of token m: two rotary pairs of one head
+            const int n = n0 + fg * 4;
+            if (n >= N) continue;
+            const int hd = ex.hd, head = n / hd, d = n - head * hd;
+            const int pos = ex.tok_pos[m];
+            float v[4] = {acc[0][ct][0], acc[0][ct][1], acc[0][ct][2], acc[0][ct][3]};
+            if (head < ex.H + ex.Hkv) {
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    const int dd = d + 2 * pr;
+                    if (dd < ex.rot) {
+                        float sn, cs;
+                        sincosf((float)pos * ex.freqs[dd >> 1], &sn, &cs);
+                        const float a = v[2 * pr], bb = v[2 * pr + 1];
+                        v[2 * pr] = a * cs - bb * sn;
+                        v[2 * pr + 1] = bb * cs + a * sn;
+                    }
+                }
+            }
+            Frag8 pk;
+            bf16_t* e = (bf16_t*)&pk.u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) e[j] = float_to_bf16(v[j]);
+            if (head < ex.H) {
+                *(uint2*)(ex.q_out + ((size_t)m * ex.H + head) * hd + d) = make_uint2(pk.u.x, pk.u.y);
+            } else if (ex.k_pages) {
+                const int page = ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + pos / GFA_PAGE];
+                const int off = pos % GFA_PAGE;
+                if (head < ex.H + ex.Hkv) {
+                    *(uint2*)(ex.k_pages + page_row(page, head - ex.H, off, ex.Hkv, hd) + d) =
+                        make_uint2(pk.u.x, pk.u.y);
+                } else {
+                    const int g = head - ex.H - ex.Hkv;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        ex.v_pages[value_elem(page, g, d + j, off, ex.Hkv, hd)] = e[j];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + fg * 4 + j;
+                if (n < N) skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
+            }
         }
     }
 }
 
-template <int MODE>
+template <int MODE, bool NORM>
 static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
-                              int ldo, int gate_rows, hipStream_t stream) {
+                              int ldo, int gate_rows, const SkinnyExtra& ex, hipStream_t stream) {
     constexpr int RT = (MODE == 3) ? 2 : 1;
     const int tiles = (N + 15) / 16;
     const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
@@ -326,14 +466,36 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     const int nw_max = (MODE == 3) ? 4 : 8;
     while (nw < nw_max && tiles * nw < 2048 && pieces >= 4 * nw) nw *= 2;
     size_t shmem = (size_t)nw * RT * SM_TILE;
-    const size_t red = (size_t)nw * RT * ct * 64 * sizeof(floatx4_t);
+    const size_t red = (size_t)nw * RT * ct * 64 * sizeof(floatx4_t) + (size_t)nw * ct * 16 * sizeof(float);
     if (nw > 1 && red > shmem) shmem = red;
-    switch (ct) {
-        case 1: skinny_mfma_kernel<1, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows); break;
-        case 2: skinny_mfma_kernel<2, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows); break;
-        case 3: skinny_mfma_kernel<3, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows); break;
-        default: skinny_mfma_kernel<4, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows); break;
+    while (shmem > 96 * 1024 && nw > 1) {                // keep two workgroups per compute unit
+        nw /= 2;
+        shmem = (size_t)nw * RT * SM_TILE;
+        const size_t r2 = (size_t)nw * RT * ct * 64 * sizeof(floatx4_t) + (size_t)nw * ct * 16 * sizeof(float);
+        if (nw > 1 && r2 > shmem) shmem = r2;
     }
+#define GFA_LAUNCH_MFMA(CTV)                                                                      \
+    do {                                                                                          \
+        static bool raised = false;                                                               \
+        if (!raised) {                                                                            \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, NORM>,                 \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
+            raised = true;                                                                        \
+        }                                                                                         \
+        skinny_mfma_kernel<CTV, MODE, NORM><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, ex); \
+    } while (0)
+    if (NORM) {                                          // the fused norm serves one 16-row tile
+        if (ct != 1) return (int)hipErrorInvalidValue;
+        GFA_LAUNCH_MFMA(1);
+    } else {
+        switch (ct) {
+            case 1: GFA_LAUNCH_MFMA(1); break;
+            case 2: GFA_LAUNCH_MFMA((NORM ? 1 : 2)); break;
+            case 3: GFA_LAUNCH_MFMA((NORM ? 1 : 3)); break;
+            default: GFA_LAUNCH_MFMA((NORM ? 1 : 4)); break;
+        }
+    }
+#undef GFA_LAUNCH_MFMA
     return GFA_LAUNCH_RESULT();
 }
 
@@ -343,13 +505,64 @@ extern "C" int gfa_skinny_mfma_bf16(const void* x, const void* w, void* out, int
     if (M > 64 || K <= 0 || K % 8 != 0) return (int)hipErrorInvalidValue;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
+    SkinnyExtra ex = {};
     switch (mode) {
-        case 0: return launch_skinny_mfma<0>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
-        case 1: return launch_skinny_mfma<1>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
-        case 2: return launch_skinny_mfma<2>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
-        case 3: return launch_skinny_mfma<3>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
+        case 0: return launch_skinny_mfma<0, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 1: return launch_skinny_mfma<1, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 2: return launch_skinny_mfma<2, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 3: return launch_skinny_mfma<3, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
     }
     return (int)hipErrorInvalidValue;
+}
+
+// The same products reading the float residual stream through an RMS norm
+// (x_f32 [M, K], norm_w [K]): modes 0, 1 and 3 as above.
+extern "C" int gfa_skinny_norm_bf16(const float* x_f32, const float* norm_w, float eps, const void* w,
+                                    void* out, int M, int N, int K, int ldo, int mode,
+                                    int gate_rows, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0) return (int)hipErrorInvalidValue;
+    const bf16_t* wp = (const bf16_t*)w;
+    SkinnyExtra ex = {};
+    ex.x_f32 = x_f32;
+    ex.norm_w = norm_w;
+    ex.eps = eps;
+    switch (mode) {
+        case 0: return launch_skinny_mfma<0, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 1: return launch_skinny_mfma<1, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 3: return launch_skinny_mfma<3, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+    }
+    return (int)hipErrorInvalidValue;
+}
+
+// norm -> fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
+// w [(H + 2 Hkv) hd, K]; head size a multiple of 16, rotary width even, interleaved pairs.
+extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, float eps,
+                                       const void* w, void* q_out, void* k_pages, void* v_pages,
+                                       const float* freqs, const int* tok_seq, const int* tok_pos,
+                                       const int* table, int table_stride, int M, int K, int H,
+                                       int Hkv, int hd, int rot, hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0 || hd % 16 != 0 || rot % 2 != 0 || rot > hd)
+        return (int)hipErrorInvalidValue;
+    SkinnyExtra ex = {};
+    ex.x_f32 = x_f32;
+    ex.norm_w = norm_w;
+    ex.eps = eps;
+    ex.q_out = (bf16_t*)q_out;
+    ex.k_pages = (bf16_t*)k_pages;
+    ex.v_pages = (bf16_t*)v_pages;
+    ex.freqs = freqs;
+    ex.tok_seq = tok_seq;
+    ex.tok_pos = tok_pos;
+    ex.table = table;
+    ex.table_stride = table_stride;
+    ex.H = H;
+    ex.Hkv = Hkv;
+    ex.hd = hd;
+    ex.rot = rot;
+    const int N = (H + 2 * Hkv) * hd;
+    return launch_skinny_mfma<4, true>(nullptr, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
 }
 
 // x [M, K], w [N, K] (gate mode: [2 * N, K], gate_rows = N), out [M, ldo].

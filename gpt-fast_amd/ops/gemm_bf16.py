@@ -88,3 +88,85 @@ def wide_f32_out(x: torch.Tensor, w: torch.Tensor):
         for n0 in range(0, w.shape[0], step):
             out[:, n0:n0 + step] = xf @ w[n0:n0 + step].float().t()
         return out
+
+
+def _check_normed(x_f32, norm_w, w, what):
+    require_device(x_f32, norm_w, w)
+    require_contiguous(x=x_f32, norm_w=norm_w, w=w)
+    if x_f32.dtype != torch.float32 or norm_w.dtype != torch.float32 or w.dtype != torch.bfloat16:
+        raise KernelError(f"{what}: x and the norm weight must be float32, w bfloat16")
+    if x_f32.dim() != 2 or w.dim() != 2 or x_f32.shape[1] != w.shape[1] \
+            or norm_w.numel() != w.shape[1]:
+        raise KernelError(f"{what}: x {tuple(x_f32.shape)}, norm {tuple(norm_w.shape)} and "
+                          f"w {tuple(w.shape)} do not fit")
+    if not 0 < x_f32.shape[0] <= 16 or w.shape[1] % 8:
+        raise KernelError(f"{what}: takes 1..16 rows and an inner size that is a multiple of 8")
+
+
+def can_fuse_norm(n_rows: int, inner: int) -> bool:
+    # beyond one 16-row tile the float32 reads of x outweigh the saved norm kernel
+    return 0 < n_rows <= 16 and inner % 8 == 0
+
+
+def skinny_normed(x_f32, norm_w, eps: float, w, out_dtype=torch.bfloat16):
+    """rmsnorm(x_f32; norm_w, eps) times w transposed, one kernel: [M, N] in out_dtype."""
+    _check_normed(x_f32, norm_w, w, "skinny_normed")
+    M, K = x_f32.shape
+    N = w.shape[0]
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"skinny_normed: output type {out_dtype}")
+    out = torch.empty((M, N), dtype=out_dtype, device=w.device)
+    check(library("gemm_bf16").gfa_skinny_norm_bf16(
+        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(w), ptr(out), _i(M), _i(N), _i(K), _i(N),
+        _i(0 if out_dtype == torch.bfloat16 else 1), _i(0), stream_handle()), "skinny_normed")
+    return out
+
+
+def skinny_normed_gated(x_f32, norm_w, eps: float, w13):
+    """silu(n W1^T) * (n W3^T) with n = rmsnorm(x_f32), one kernel: bfloat16 [M, I]."""
+    _check_normed(x_f32, norm_w, w13, "skinny_normed_gated")
+    M, K = x_f32.shape
+    if w13.shape[0] % 2:
+        raise KernelError("skinny_normed_gated: w13 needs an even number of rows")
+    I = w13.shape[0] // 2
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
+    check(library("gemm_bf16").gfa_skinny_norm_bf16(
+        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I), _i(K),
+        _i(I), _i(3), _i(I), stream_handle()), "skinny_normed_gated")
+    return out
+
+
+def qkv_rope_store(x_f32, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, k_pages,
+                   v_pages, n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int):
+    """Norm, fused q/k/v projection, rotation of interleaved pairs and the cache write in
+    one kernel; returns q [M, H, hd].  k_pages None: keys and values are not stored."""
+    _check_normed(x_f32, norm_w, wqkv, "qkv_rope_store")
+    M, K = x_f32.shape
+    if wqkv.shape[0] != (n_heads + 2 * n_kv_heads) * head_dim:
+        raise KernelError("qkv_rope_store: wqkv does not have (H + 2 Hkv) * hd rows")
+    if head_dim % 16 or rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+        raise KernelError("qkv_rope_store: head_dim must be a multiple of 16, rotary_dim even")
+    require_device(freqs, tok_seq, tok_pos, table, k_pages, v_pages)
+    if rotary_dim and (freqs is None or freqs.numel() != rotary_dim // 2
+                       or freqs.dtype != torch.float32):
+        raise KernelError("qkv_rope_store: one float32 frequency per rotary pair")
+    for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos), ("table", table)):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise KernelError(f"qkv_rope_store: {name} must be contiguous int32")
+    if tok_seq.numel() < M or tok_pos.numel() < M:
+        raise KernelError("qkv_rope_store: token maps are shorter than the batch")
+    if (k_pages is None) != (v_pages is None):
+        raise KernelError("qkv_rope_store: give both k_pages and v_pages, or neither")
+    if k_pages is not None:
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, 64, head_dim) \
+                or tuple(v_pages.shape[1:]) != (n_kv_heads, head_dim, 64) \
+                or k_pages.dtype != torch.bfloat16 or v_pages.dtype != torch.bfloat16 \
+                or not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelError("qkv_rope_store: pages have the wrong shape or dtype")
+    q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=wqkv.device)
+    check(library("gemm_bf16").gfa_qkv_rope_store_bf16(
+        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(wqkv), ptr(q), ptr(k_pages),
+        ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table), _i(table.shape[1]),
+        _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim), _i(rotary_dim), stream_handle()),
+        "qkv_rope_store")
+    return q

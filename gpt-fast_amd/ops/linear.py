@@ -57,3 +57,26 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
     if x.shape[0] <= SKINNY_MAX_ROWS:
         return _fast().skinny_gated(x, w13)
     return K.silu_mul(torch.matmul(x, w13.t()))
+
+
+# ----------------------------------------------------------------------------- fused with the norm
+def can_fuse_norm(residual: torch.Tensor, norm, w: torch.Tensor) -> bool:
+    """True if the few-row kernels can read ``residual`` through ``norm`` themselves: a
+    bfloat16 engine, an RMS norm, at most 64 rows, an inner size that is a multiple of 8."""
+    return (w.dtype == torch.bfloat16 and getattr(getattr(norm, "spec", None), "kind", None) == "rms"
+            and getattr(norm, "weight", None) is not None
+            and _fast().can_fuse_norm(residual.shape[0], w.shape[1]))
+
+
+def gated_linear_normed(residual, norm_w, eps, w13):
+    return _fast().skinny_normed_gated(residual, norm_w, eps, w13)
+
+
+def linear_normed(residual, norm_w, eps, w, out_dtype=torch.bfloat16):
+    return _fast().skinny_normed(residual, norm_w, eps, w, out_dtype=out_dtype)
+
+
+def qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
+                   n_heads, n_kv_heads, head_dim, rotary_dim):
+    return _fast().qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table,
+                                  k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotary_dim)

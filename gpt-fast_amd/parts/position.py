@@ -10,6 +10,7 @@ import torch
 
 from ..config.spec import PositionSpec
 from ..ops import kernels as K
+from ..ops import linear as L
 from .base import Part, Runtime, register_position
 
 
@@ -68,6 +69,19 @@ class RotaryPosition(Part):
             entry.k_pages if write else None, entry.v_pages if write else None,
             n_heads, n_kv_heads, head_dim, self.spec.rotary_dim,
             self.LAYOUTS[self.spec.layout])
+
+
+    def project_rotate_store(self, residual, norm, wqkv, batch, entry, n_heads, n_kv_heads,
+                             head_dim):
+        """Norm + projection + rotation + cache write in one kernel (interleaved pairs
+        only: both elements of a pair are then in one lane).  None: not available."""
+        if self.spec.layout != "interleaved":
+            return None
+        write = entry is not None and entry.writes
+        return L.qkv_rope_store(
+            residual, norm.weight, norm.spec.eps, wqkv, self.freqs, batch.tok_seq, batch.tok_pos,
+            batch.table(entry.group_id), entry.k_pages if write else None,
+            entry.v_pages if write else None, n_heads, n_kv_heads, head_dim, self.spec.rotary_dim)
 
 
 class NoPosition(Part):

@@ -301,3 +301,54 @@ def test_argmax_and_sampling():
     assert torch.equal(b, a[order.cpu()])
     c = sample(logits, SamplingParams(temperature=1.0, top_k=100, seed=6), keys, pos, 1).cpu()
     assert not torch.equal(a, c)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K_,eps", [(48, 64, 1e-5), (208, 200, 1e-6), (1024, 4096, 1e-5)])
+def test_products_fused_with_the_norm(M, N, K_, eps):
+    from gpt_fast_amd.ops import gemm_bf16 as G
+    torch.manual_seed(8)
+    x = torch.randn(M, K_, device=DEV) * 2
+    g = 1 + 0.1 * torch.randn(K_, device=DEV)
+    w = bf(torch.randn(N, K_, device=DEV) * 0.1)
+    n = x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * g.double()
+    ref = n @ w.double().T
+    close(G.skinny_normed(x, g, eps, w, out_dtype=torch.float32), ref, 1e-2)
+    close(G.skinny_normed(x, g, eps, w), ref, 1.5e-2)
+    I = N // 2
+    a = ref[:, :I]
+    close(G.skinny_normed_gated(x, g, eps, w), (a * torch.sigmoid(a)) * ref[:, I:], 2e-2)
+    # against the unfused kernels of the engine: same operands up to one rounding of x
+    unfused = G.skinny(K().rmsnorm(x, g, eps, torch.bfloat16), w, out_dtype=torch.float32)
+    close(G.skinny_normed(x, g, eps, w, out_dtype=torch.float32), unfused, 1e-2)
+
+
+@pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])
+def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
+    from gpt_fast_amd.ops import gemm_bf16 as G
+    torch.manual_seed(9)
+    D = 72 if hd < 128 else 512
+    pos = [0, 5, 63, 64, 200, 3000]
+    seq = [1, 0, 1, 0, 1, 0]                      # two sequences with tables of their own
+    M = len(pos)
+    x = torch.randn(M, D, device=DEV)
+    g = 1 + 0.1 * torch.randn(D, device=DEV)
+    w = bf(torch.randn((H + 2 * G_) * hd, D, device=DEV) * 0.1)
+    freqs = (1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV) if rot else None
+    table = torch.stack([torch.randperm(50)[:48], torch.randperm(50)[:48] + 50]).to(torch.int32).to(DEV)
+    tok_seq = torch.tensor(seq, dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    kp = torch.zeros(100, G_, 64, hd, device=DEV, dtype=torch.bfloat16)
+    vp = torch.zeros(100, G_, hd, 64, device=DEV, dtype=torch.bfloat16)
+    q = G.qkv_rope_store(x, g, 1e-5, w, freqs, tok_seq, tok_pos, table, kp, vp, H, G_, hd, rot)
+    # the unfused chain of the same engine
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    qkv = G.skinny(K().rmsnorm(x, g, 1e-5, torch.bfloat16), w)
+    q2 = K().rope_cache_write(qkv, freqs, tok_seq, tok_pos, table, kp2, vp2, H, G_, hd, rot, 0)
+    close(q, q2, 1.5e-2)
+    close(kp, kp2, 1.5e-2)
+    close(vp, vp2, 1.5e-2)
+    assert torch.equal(kp == 0, kp2 == 0) and torch.equal(vp == 0, vp2 == 0)   # same places written
+    # no pages: q only
+    q3 = G.qkv_rope_store(x, g, 1e-5, w, freqs, tok_seq, tok_pos, table, None, None, H, G_, hd, rot)
+    assert torch.equal(q3, q)

@@ -56,10 +56,15 @@ class KVGroup:
         self.n_pages = n_pages
         # keys as rows [PAGE, head_dim]; values transposed [head_dim, PAGE]: the operand
         # layouts of the matrix-core attention kernel
-        self.k = torch.empty((entries, n_pages, need.n_kv_heads, PAGE, need.head_dim),
+        # one page beyond the pool (index n_pages) belongs to no sequence: rows of a batch
+        # that only fill a fixed shape are pointed at it
+        self.k = torch.empty((entries, n_pages + 1, need.n_kv_heads, PAGE, need.head_dim),
                              dtype=dtype, device=device)
-        self.v = torch.empty((entries, n_pages, need.n_kv_heads, need.head_dim, PAGE),
+        self.v = torch.empty((entries, n_pages + 1, need.n_kv_heads, need.head_dim, PAGE),
                              dtype=dtype, device=device)
+        self.spare_page = n_pages
+        self.k[:, n_pages].zero_()
+        self.v[:, n_pages].zero_()
         self.pages = FreeList(n_pages, "cache page")
         self.held: Dict[int, List[int]] = {}      # slot -> page of each PAGE tokens, -1 = given back
 

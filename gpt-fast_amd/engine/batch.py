@@ -29,7 +29,9 @@ from ..cache.store import Cache, pages_for
 @dataclass
 class Entry:
     """One sequence's share of a step: its slot, its new tokens, and the indices among
-    these tokens whose logits are wanted."""
+    these tokens whose logits are wanted.  ``slot`` None marks a row that belongs to no
+    sequence and only keeps a captured batch's shape: it reads and writes the cache's
+    spare page and its results are ignored."""
     slot: int
     tokens: Sequence[int]
     want: Sequence[int] = ()
@@ -108,7 +110,7 @@ def fill_host(layout: BatchLayout, host: np.ndarray, entries: Sequence[Entry],
         host[p0:p0 + q] = np.arange(start, start + q, dtype=np.int32)
         host[f["q_start"][0] + b] = n
         host[f["start_pos"][0] + b] = start
-        host[f["slots"][0] + b] = e.slot
+        host[f["slots"][0] + b] = -1 if e.slot is None else e.slot
         host[f["row_keys"][0] + b] = e.key
         for i in e.want:
             if not 0 <= i < q:
@@ -121,8 +123,11 @@ def fill_host(layout: BatchLayout, host: np.ndarray, entries: Sequence[Entry],
         for gid, (off, _) in layout.tables.items():
             width = layout.table_widths[gid]
             for b, e in enumerate(entries):
-                pages = cache.page_list(gid, e.slot)
                 row = host[off + b * width: off + (b + 1) * width]
+                if e.slot is None:                    # a row that only fills the batch's shape
+                    row[:] = cache.groups[gid].spare_page
+                    continue
+                pages = cache.page_list(gid, e.slot)
                 row[:len(pages)] = pages
                 row[len(pages):] = -1
 

@@ -69,6 +69,37 @@ class BatchRun:
         if self.callback is not None:
             self.callback(rows, [int(t) for t in tokens])
 
+    def _decode_in_session(self) -> None:
+        """One-token steps through a session that keeps the drawn tokens on the device.
+        A step is launched before the tokens of the step before it are read, so a stop
+        token is noticed one step late; what that step drew for the ended request is
+        dropped.  Requests that end by length are known beforehand and are not launched."""
+        rows = self.live()
+        session = self.stepper.open_session(
+            [self.slots[i] for i in rows], [self.keys[i] for i in rows],
+            [self.new[i][-1] for i in rows], self.max_new - 1)
+        launched = {i: len(self.new[i]) for i in rows}       # tokens drawn or under way
+        pending = None
+        while True:
+            active = [i for i in rows if self.reason[i] is None and launched[i] < self.max_new]
+            handle = None
+            if active:
+                for r, i in enumerate(rows):
+                    if self.reason[i] is not None and session.slots[r] is not None:
+                        session.retire(r)
+                handle = (active, session.launch())
+                for i in active:
+                    launched[i] += 1
+                self.steps += 1
+            if pending is not None:
+                was_active, h = pending
+                tokens = session.collect(h)
+                keep = [i for i in was_active if self.reason[i] is None]
+                self._take(keep, [tokens[rows.index(i)] for i in keep])
+            pending = handle
+            if pending is None:
+                break
+
     def run(self):
         try:
             for i in range(len(self.prompts)):
@@ -78,6 +109,8 @@ class BatchRun:
                              key=self.keys[i]) for i in rows]
             self._take(rows, self.stepper.next_tokens(entries))       # generate.py:180
             self.steps = 1
+            if self.live() and hasattr(self.stepper, "open_session"):
+                self._decode_in_session()
             while True:
                 rows = self.live()
                 if not rows:
@@ -97,9 +130,10 @@ class BatchRun:
 class EngineStepper:
     """Drives an :class:`~.step.Engine` and a sampler for :class:`BatchRun`."""
 
-    def __init__(self, engine, params: SamplingParams):
+    def __init__(self, engine, params: SamplingParams, use_graph: bool = True):
         self.engine = engine
         self.params = params
+        self.use_graph = use_graph
         self.prefill_seconds = 0.0
         self.decode_seconds = 0.0
         self.decode_steps = 0
@@ -129,6 +163,44 @@ class EngineStepper:
         return out
 
 
+    def open_session(self, slots, keys, last_tokens, max_new_tokens):
+        import torch
+        from .decode import DecodeSession
+        first = torch.tensor(list(last_tokens), dtype=torch.int32, device=self.engine.rt.device)
+        return _TimedSession(DecodeSession(self.engine, slots, keys, first, self.params,
+                                           use_graph=self.use_graph,
+                                           max_new_tokens=max_new_tokens), self)
+
+
+class _TimedSession:
+    """A decode session that books its time to the stepper's counters."""
+
+    def __init__(self, session, stepper):
+        self.session = session
+        self.stepper = stepper
+        self.t_last = None
+
+    @property
+    def slots(self):
+        return self.session.slots
+
+    def retire(self, row):
+        self.session.retire(row)
+
+    def launch(self):
+        if self.t_last is None:
+            self.t_last = time.perf_counter()
+        return self.session.launch()
+
+    def collect(self, handle):
+        out = self.session.collect(handle)
+        now = time.perf_counter()
+        self.stepper.decode_seconds += now - self.t_last
+        self.stepper.decode_steps += 1
+        self.t_last = now
+        return out
+
+
 def split_batches(n_requests: int, batch_size: Optional[int]) -> List[List[int]]:
     if batch_size is None or batch_size >= n_requests:
         return [list(range(n_requests))] if n_requests else []
@@ -142,20 +214,21 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_new_tokens: int, *,
              temperature: float = 0.8, top_k: Optional[int] = None,
              stop_tokens: Optional[Sequence[int]] = None, seed: int = 1234,
              batch_size: Optional[int] = None, callback: Optional[Callable] = None,
-             stepper=None) -> GenerationResult:
+             use_graph: bool = True, stepper=None) -> GenerationResult:
     """Generate up to ``max_new_tokens`` tokens for every prompt (lists of token ids).
 
     ``temperature`` and ``top_k`` mean what they mean in the reference's ``generate``
     (generate.py:44-57); ``temperature=0`` is greedy.  ``stop_tokens`` defaults to the
     model's end-of-sequence ids (none if the configuration names none).  ``batch_size``
     bounds how many requests run together; the rest follow in further batches.
+    ``use_graph`` replays the one-token step as a captured HIP graph.
     ``callback(rows, tokens)`` is called after every step with the indices of the
     requests that drew a token and the tokens (the reference calls back per step too,
     generate.py:79)."""
     params = SamplingParams(temperature=temperature, top_k=top_k, seed=seed)
     if stop_tokens is None:
         stop_tokens = engine.model.plan.stop_tokens
-    stepper = stepper or EngineStepper(engine, params)
+    stepper = stepper or EngineStepper(engine, params, use_graph=use_graph)
     tokens: List[List[int]] = [[] for _ in prompts]
     reasons: List[str] = ["length"] * len(prompts)
     steps = 0

@@ -54,8 +54,8 @@ def test_groups_by_need():
     assert len(c.groups) == 3
     assert c.entries[0].group_id == c.entries[2].group_id != c.entries[1].group_id
     assert (c.entries[0].index, c.entries[2].index) == (0, 1)
-    assert c.groups[c.entries[0].group_id].k.shape == (2, 6, 2, 64, 8)
-    assert c.groups[c.entries[0].group_id].v.shape == (2, 6, 2, 8, 64)
+    assert c.groups[c.entries[0].group_id].k.shape == (2, 7, 2, 64, 8)       # 6 pages and the spare one
+    assert c.groups[c.entries[0].group_id].v.shape == (2, 7, 2, 8, 64)
     assert c.entries[3].state.shape == (4, 3)
     # a borrowed entry reads the lender's storage and does not write
     b = Cache([KVNeed(1, 8), KVNeed(1, 8)], [None, 0], max_tokens=64, max_sequences=1,
@@ -227,3 +227,62 @@ def test_batches_one_after_another_reuse_slots():
     assert res.finish_reasons == ["length"] * 5 and res.stats["steps"] == 9
     assert seen[0] == ([0, 1], [0, 1]) and seen[3] == ([2, 3], [2, 3]) and seen[-1] == ([4], [4])
     assert st.slots.held == 0
+
+
+class SessionStepper(ScriptedStepper):
+    """A scripted stepper that also offers decode sessions, answering one step late like
+    the device session does."""
+
+    def open_session(self, slots, keys, last_tokens, max_new_tokens):
+        outer = self
+
+        class Session:
+            def __init__(self):
+                self.slots = list(slots)
+                self.keys = list(keys)
+                self.last = list(last_tokens)
+                self.launches = 0
+
+            def retire(self, row):
+                assert self.slots[row] is not None
+                self.slots[row] = None
+
+            def launch(self):
+                self.launches += 1
+                out = []
+                for r, s in enumerate(self.slots):
+                    if s is None:
+                        out.append(-777)               # junk of a filler row
+                        continue
+                    outer.fed[s].append(self.last[r])
+                    self.last[r] = outer.script(self.keys[r], outer.fed[s])
+                    out.append(self.last[r])
+                return out
+
+            def collect(self, handle):
+                return handle
+        self.session = Session()
+        return self.session
+
+
+def test_loop_with_a_session_notices_stops_one_step_late():
+    st = SessionStepper(lambda key, fed: fed[-1] + 1)
+    prompts = [[10, 11], [47], [30, 31, 32], [49]]
+    run = BatchRun(st, prompts, keys=[0, 1, 2, 3], max_new_tokens=5, stop_tokens=[50])
+    new, why = run.run()
+    # the same tokens and reasons as the synchronous loop
+    assert new == [[12, 13, 14, 15, 16], [48, 49, 50], [33, 34, 35, 36, 37], [50]]
+    assert why == ["length", "stop", "length", "stop"]
+    assert st.slots.held == 0
+    # request 3 ended in the prefill and never entered the session; requests 0 and 2 end
+    # by length and are not launched beyond it: 4 decode steps in all
+    assert len(st.session.slots) == 3 and st.session.launches == 4
+    # request 1's filler row was retired after its stop token was seen
+    assert st.session.slots == [0, None, 2] or st.session.slots[1] is None
+
+
+def test_loop_with_a_session_single_token_budget():
+    st = SessionStepper(lambda key, fed: 7)
+    new, why = BatchRun(st, [[1, 2], [3]], [0, 1], max_new_tokens=1).run()
+    assert new == [[7], [7]] and why == ["length", "length"]
+    assert not hasattr(st, "session")                 # nothing left to decode

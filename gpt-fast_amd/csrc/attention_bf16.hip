@@ -135,36 +135,50 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
                 for (int e = 0; e < 8; ++e)
                     if (key0 + (e >> 2) * 16 + (e & 3) > pmax) vf[dt].e[e] = 0;
         }
+        // blocks wholly below every row's position (and inside every window) need no mask
+        const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             float sv[8];
             float mx = -INFINITY;
-            const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
+            if (masked) {
+                const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int key = key0 + (e >> 2) * 16 + (e & 3);
-                const float v = s[rt][e >> 2][e & 3] * scale_log2;
-                sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
-                mx = fmaxf(mx, sv[e]);
+                for (int e = 0; e < 8; ++e) {
+                    const int key = key0 + (e >> 2) * 16 + (e & 3);
+                    const float v = s[rt][e >> 2][e & 3] * scale_log2;
+                    sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
+                    mx = fmaxf(mx, sv[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    sv[e] = s[rt][e >> 2][e & 3] * scale_log2;
+                    mx = fmaxf(mx, sv[e]);
+                }
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m[rt], mx);
-            const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[rt] - m_new);
+            // a row without any key so far keeps m = -inf: exp2(-inf - -inf) must not be formed
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_safe);
             Frag pf;
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = (sv[e] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sv[e] - m_new);
+                const float p = __builtin_amdgcn_exp2f(sv[e] - m_safe);      // 2^-inf = 0
                 sum += p;
                 pf.e[e] = float_to_bf16(p);
             }
             l[rt] = l[rt] * alpha + sum;
             m[rt] = m_new;
+            // the running maximum rarely moves after the first blocks: skip the rescale then
+            const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 if (dt * 16 < hd) {
-                    o[rt][dt] *= alpha;
+                    if (rescale) o[rt][dt] *= alpha;
                     o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
                 }
             }

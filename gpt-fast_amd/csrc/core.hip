@@ -54,8 +54,8 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
 
 // The same for rows of up to 1024 * VPT elements (a multiple of 4): the row is read once
 // with 16-byte loads, kept in registers between the sum and the scaling.
-template <typename T, int VPT>
-__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
+template <typename T, int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(
         const float* __restrict__ x, const float* __restrict__ w, const int* __restrict__ rows,
         T* __restrict__ out, int dim, float eps) {
     __shared__ float scratch[16];
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
-        const int idx = threadIdx.x + j * 256;
+        const int idx = threadIdx.x + j * THREADS;
         v[j] = idx < n4 ? xr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
         ss = fmaf(v[j].x, v[j].x, ss);
         ss = fmaf(v[j].y, v[j].y, ss);
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
     T* o = out + (size_t)i * dim;
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
-        const int idx = threadIdx.x + j * 256;
+        const int idx = threadIdx.x + j * THREADS;
         if (idx < n4) {
             const float4 g = w4[idx];
             store_from_float(o + 4 * idx + 0, v[j].x * rs * g.x);
@@ -95,10 +95,10 @@ template <typename T>
 static bool launch_rmsnorm_vec(const float* x, const float* w, const int* rows, T* out, int n_rows,
                                int dim, float eps, hipStream_t stream) {
     if (dim % 4 != 0 || dim > 8192) return false;
-    if (dim <= 1024) rmsnorm_vec_kernel<T, 1><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
-    else if (dim <= 2048) rmsnorm_vec_kernel<T, 2><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
-    else if (dim <= 4096) rmsnorm_vec_kernel<T, 4><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
-    else rmsnorm_vec_kernel<T, 8><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    // one float4 per thread where the row allows it: the kernel is a chain of latencies
+    if (dim <= 1024) rmsnorm_vec_kernel<T, 1, 256><<<n_rows, 256, 0, stream>>>(x, w, rows, out, dim, eps);
+    else if (dim <= 4096) rmsnorm_vec_kernel<T, 1, 1024><<<n_rows, 1024, 0, stream>>>(x, w, rows, out, dim, eps);
+    else rmsnorm_vec_kernel<T, 2, 1024><<<n_rows, 1024, 0, stream>>>(x, w, rows, out, dim, eps);
     return true;
 }
 

@@ -537,13 +537,15 @@ extern "C" int gfa_skinny_norm_bf16(const float* x_f32, const float* norm_w, flo
 
 // norm -> fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
 // w [(H + 2 Hkv) hd, K]; head size a multiple of 16, rotary width even, interleaved pairs.
+// Either x_f32 with its norm (x_bf16 null), or x_bf16 already normed (up to 64 rows).
 extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, float eps,
+                                       const void* x_bf16,
                                        const void* w, void* q_out, void* k_pages, void* v_pages,
                                        const float* freqs, const int* tok_seq, const int* tok_pos,
                                        const int* table, int table_stride, int M, int K, int H,
                                        int Hkv, int hd, int rot, hipStream_t stream) {
     if (M <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 8 != 0 || hd % 16 != 0 || rot % 2 != 0 || rot > hd)
+    if (M > (x_bf16 ? 64 : 16) || K <= 0 || K % 8 != 0 || hd % 16 != 0 || rot % 2 != 0 || rot > hd)
         return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.x_f32 = x_f32;
@@ -562,6 +564,8 @@ extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, 
     ex.hd = hd;
     ex.rot = rot;
     const int N = (H + 2 * Hkv) * hd;
+    if (x_bf16)
+        return launch_skinny_mfma<4, false>((const bf16_t*)x_bf16, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
     return launch_skinny_mfma<4, true>(nullptr, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
 }
 

@@ -136,12 +136,20 @@ def skinny_normed_gated(x_f32, norm_w, eps: float, w13):
     return out
 
 
-def qkv_rope_store(x_f32, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, k_pages,
+def qkv_rope_store(x, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, k_pages,
                    v_pages, n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int):
-    """Norm, fused q/k/v projection, rotation of interleaved pairs and the cache write in
-    one kernel; returns q [M, H, hd].  k_pages None: keys and values are not stored."""
-    _check_normed(x_f32, norm_w, wqkv, "qkv_rope_store")
-    M, K = x_f32.shape
+    """Fused q/k/v projection, rotation of interleaved pairs and the cache write in one
+    kernel; returns q [M, H, hd].  ``x`` is either the float32 residual stream, read
+    through the RMS norm (``norm_w``, ``eps``; up to 16 rows), or bfloat16 rows that are
+    normed already (``norm_w`` None; up to 64 rows).  k_pages None: nothing is stored."""
+    fused_norm = x.dtype == torch.float32
+    if fused_norm:
+        _check_normed(x, norm_w, wqkv, "qkv_rope_store")
+    else:
+        _check_operands(x, wqkv, "qkv_rope_store")
+        if wqkv.shape[1] % 8:
+            raise KernelError("qkv_rope_store: the inner size must be a multiple of 8")
+    M, K = x.shape
     if wqkv.shape[0] != (n_heads + 2 * n_kv_heads) * head_dim:
         raise KernelError("qkv_rope_store: wqkv does not have (H + 2 Hkv) * hd rows")
     if head_dim % 16 or rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
@@ -165,8 +173,9 @@ def qkv_rope_store(x_f32, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, tab
             raise KernelError("qkv_rope_store: pages have the wrong shape or dtype")
     q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=wqkv.device)
     check(library("gemm_bf16").gfa_qkv_rope_store_bf16(
-        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(wqkv), ptr(q), ptr(k_pages),
-        ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table), _i(table.shape[1]),
-        _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim), _i(rotary_dim), stream_handle()),
-        "qkv_rope_store")
+        ptr(x if fused_norm else None), ptr(norm_w if fused_norm else None),
+        ctypes.c_float(eps if fused_norm else 0.0), ptr(None if fused_norm else x), ptr(wqkv),
+        ptr(q), ptr(k_pages), ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table),
+        _i(table.shape[1]), _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim),
+        _i(rotary_dim), stream_handle()), "qkv_rope_store")
     return q

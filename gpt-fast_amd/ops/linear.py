@@ -68,6 +68,12 @@ def can_fuse_norm(residual: torch.Tensor, norm, w: torch.Tensor) -> bool:
             and _fast().can_fuse_norm(residual.shape[0], w.shape[1]))
 
 
+def can_project_rotate_store(x: torch.Tensor, wqkv: torch.Tensor, head_dim: int) -> bool:
+    """True if the fused projection / rotation / cache-write kernel takes these rows."""
+    return (x.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
+            and wqkv.shape[1] % 8 == 0 and head_dim % 16 == 0)
+
+
 def gated_linear_normed(residual, norm_w, eps, w13):
     return _fast().skinny_normed_gated(residual, norm_w, eps, w13)
 

@@ -41,27 +41,18 @@ class Attention(Part):
 
     def forward(self, x, batch, entry, residual):
         s = self.spec
-        qkv = L.linear(x, self.wqkv)                                        # model.py:195
-        q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
-                                           s.head_dim)                      # model.py:201-207
+        q = None
+        fused = getattr(self.position, "project_rotate_store", None)
+        if fused is not None and L.can_project_rotate_store(x, self.wqkv, s.head_dim):
+            # few rows: projection, rotation and cache write in one kernel
+            q = fused(x, self.wqkv, batch, entry, s.n_heads, s.n_kv_heads, s.head_dim)
+        if q is None:
+            qkv = L.linear(x, self.wqkv)                                    # model.py:195
+            q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
+                                               s.head_dim)                  # model.py:201-207
         y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
                         self.scale, self.window)                            # model.py:209-211
         L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual)  # :215, 162
-
-    def forward_normed(self, residual, norm, batch, entry) -> bool:
-        """Few rows in bfloat16: norm, projection, rotation and cache write are one kernel
-        if the position encoding offers it."""
-        s = self.spec
-        fused = getattr(self.position, "project_rotate_store", None)
-        if fused is None or s.head_dim % 16 or not L.can_fuse_norm(residual, norm, self.wqkv):
-            return False
-        q = fused(residual, norm, self.wqkv, batch, entry, s.n_heads, s.n_kv_heads, s.head_dim)
-        if q is None:
-            return False
-        y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
-                        self.scale, self.window)
-        L.linear_into(y.view(residual.shape[0], s.n_heads * s.head_dim), self.wo, residual)
-        return True
 
 
 register_mixer("attention", Attention)

@@ -27,13 +27,5 @@ class GatedFeedForward(Part):
         h = L.gated_linear(x, self.w13)
         L.linear_into(h, self.w2, residual)
 
-    def forward_normed(self, residual, norm, batch) -> bool:
-        """Few rows in bfloat16: the norm runs inside the gate product's kernel."""
-        if not L.can_fuse_norm(residual, norm, self.w13):
-            return False
-        h = L.gated_linear_normed(residual, norm.weight, norm.spec.eps, self.w13)
-        L.linear_into(h, self.w2, residual)
-        return True
-
 
 register_feed_forward("gated", GatedFeedForward)

@@ -71,15 +71,14 @@ class RotaryPosition(Part):
             self.LAYOUTS[self.spec.layout])
 
 
-    def project_rotate_store(self, residual, norm, wqkv, batch, entry, n_heads, n_kv_heads,
-                             head_dim):
-        """Norm + projection + rotation + cache write in one kernel (interleaved pairs
-        only: both elements of a pair are then in one lane).  None: not available."""
+    def project_rotate_store(self, x, wqkv, batch, entry, n_heads, n_kv_heads, head_dim):
+        """Projection + rotation + cache write in one kernel for few rows (interleaved
+        pairs only: both elements of a pair are then in one lane).  None: not available."""
         if self.spec.layout != "interleaved":
             return None
         write = entry is not None and entry.writes
         return L.qkv_rope_store(
-            residual, norm.weight, norm.spec.eps, wqkv, self.freqs, batch.tok_seq, batch.tok_pos,
+            x, None, 0.0, wqkv, self.freqs, batch.tok_seq, batch.tok_pos,
             batch.table(entry.group_id), entry.k_pages if write else None,
             entry.v_pages if write else None, n_heads, n_kv_heads, head_dim, self.spec.rotary_dim)
 

@@ -352,3 +352,10 @@ def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     # no pages: q only
     q3 = G.qkv_rope_store(x, g, 1e-5, w, freqs, tok_seq, tok_pos, table, None, None, H, G_, hd, rot)
     assert torch.equal(q3, q)
+    # rows that are normed already (the engine's path): same kernel without the norm
+    kp4, vp4 = torch.zeros_like(kp), torch.zeros_like(vp)
+    xn = K().rmsnorm(x, g, 1e-5, torch.bfloat16)
+    q4 = G.qkv_rope_store(xn, None, 0.0, w, freqs, tok_seq, tok_pos, table, kp4, vp4, H, G_, hd, rot)
+    close(q4, q2, 1e-2)
+    close(kp4, kp2, 1e-2)
+    assert torch.equal(vp4, vp2)                       # values are not rotated: same products

@@ -16,8 +16,10 @@ import torch
 from . import kernels as K
 from .library import KernelError
 
-# products with at most this many rows go to the hand-written streaming kernels
-SKINNY_MAX_ROWS = 64
+# products with at most this many rows go to the hand-written streaming kernels (one 16-row
+# matrix-core tile of x); beyond that x no longer fits a wave's registers and the vendor
+# library's tiled kernels are faster (measured at 32 and 64 rows)
+SKINNY_MAX_ROWS = 16
 
 
 def _fast():

@@ -324,3 +324,35 @@ def test_toy_mixer_with_state_registers_and_steps(tmp_path_factory):
         out.append(eng.step(entries).cpu())
     assert rel_err(torch.cat(out), whole) < 1e-5
     assert not torch.isnan(whole).any() and float(whole.abs().max()) > 0
+
+
+@pytest.mark.parametrize("n_seqs", [5, 24, 40])
+def test_graph_replays_equal_eager_steps_for_any_batch_size(tmp_path_factory, n_seqs):
+    """The captured step is replayed many times with eager work and synchronisations in
+    between; every replay must give the tokens of the uncaptured step.  24 and 40 rows go
+    through the vendor library's products inside the graph."""
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.engine.decode import DecodeSession
+    from gpt_fast_amd.sampling import SamplingParams
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg = plain.read_config(folder)
+    prompts = [util.random_tokens(cfg["vocab"], 1 + (7 * i) % 50, 300 + i) for i in range(n_seqs)]
+    runs = {}
+    for use_graph in (False, True):
+        eng = engine_for(folder, "bfloat16", max_tokens=64 * 2 * n_seqs)
+        slots = [eng.start_sequence() for _ in prompts]
+        logits = eng.step([Entry(s, p, want=[len(p) - 1]) for s, p in zip(slots, prompts)])
+        first = logits.argmax(-1).to(torch.int32)
+        sess = DecodeSession(eng, slots, list(range(n_seqs)), first,
+                             SamplingParams(temperature=0.7, top_k=20, seed=3),
+                             use_graph=use_graph, max_new_tokens=24)
+        got = []
+        for step in range(20):
+            got.append(sess.collect(sess.launch()))
+            if step % 3 == 0:                       # eager work between replays
+                torch.cuda.synchronize()
+                _ = (torch.ones(1000, device="cuda:0") * 2).sum().item()
+        runs[use_graph] = got
+        for s in slots:
+            eng.end_sequence(s)
+    assert runs[True] == runs[False]

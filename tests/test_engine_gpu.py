@@ -24,7 +24,7 @@ def whole(engine, tokens):
     return logits.cpu()
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype,tol", DTYPES)
 def test_whole_prompt(tmp_path_factory, name, dtype, tol):
     folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
@@ -38,7 +38,7 @@ def test_whole_prompt(tmp_path_factory, name, dtype, tol):
         assert rel_err(got, want) < tol, (name, dtype, n)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype,tol", DTYPES)
 def test_last_32_one_by_one(tmp_path_factory, name, dtype, tol):
     from gpt_fast_amd import Entry
@@ -60,7 +60,7 @@ def test_last_32_one_by_one(tmp_path_factory, name, dtype, tol):
         assert torch.equal(got, whole(eng, tokens))
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype,tol", DTYPES)
 def test_unequal_batches_reuse_slots(tmp_path_factory, name, dtype, tol):
     from gpt_fast_amd import Entry

@@ -32,7 +32,14 @@ TINY_C = {   # odd sizes: head_dim given and != hidden/heads, GQA 5:1... width 2
     "max_position_embeddings": 512, "rope_theta": 50000.0, "rms_norm_eps": 3e-6,
     "rope_scaling": None, "tie_word_embeddings": True,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+TINY_D = {   # sizes the fast kernels refuse: width 100 (no multiple of 8), head size 20, vocab 131
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 100, "num_hidden_layers": 2, "num_attention_heads": 5,
+    "num_key_value_heads": 1, "intermediate_size": 52, "vocab_size": 131,
+    "max_position_embeddings": 256, "rope_theta": 1000.0, "rms_norm_eps": 1e-5,
+    "rope_scaling": None, "tie_word_embeddings": False,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def make_folder(tmp, name, seed=0, dtype="float32", std=0.05):

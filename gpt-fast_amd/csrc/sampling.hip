@@ -186,3 +186,230 @@ extern "C" int gfa_sample(const float* logits, size_t row_stride, int n_rows, in
         (uint32_t)(seed >> 32), row_keys, positions, position_offset, out, probs_out);
     return GFA_LAUNCH_RESULT();
 }
+
+// --------------------------------------------------------------------------------------
+// The same choices with a row spread over many workgroups, for large vocabularies: one
+// workgroup per chunk of SPL_CHUNK logits, a handful of small launches whose partial
+// results meet in a workspace.  Integer histograms are summed with atomics (the sum does
+// not depend on the order); float partials are added in chunk order.  Workspace, per row:
+//   int   hist[4][256]   (zeroed by the caller)      int   state[2] = {prefix key, remaining}
+//   float pmax[NB], psum[NB], pbest_v[NB]            int   pbest_i[NB]
+#define SPL_CHUNK 4096
+#define SPL_THREADS 1024
+
+struct SplitWs {
+    unsigned* hist;      // [B][4][256]
+    unsigned* state;     // [B][2]
+    float* pmax;         // [B][NB]
+    float* psum;         // [B][NB]
+    float* pbest_v;      // [B][NB]
+    int* pbest_i;        // [B][NB]
+    int NB;
+};
+
+__device__ __forceinline__ void split_load(const float* row, int V, int chunk, float (&v)[4], int& i0) {
+    i0 = chunk * SPL_CHUNK + threadIdx.x * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] = (i0 + c < V) ? row[i0 + c] : __builtin_nanf("");
+}
+
+// pass 0..3 of the radix select: histogram of byte (3 - pass) of the keys that match the
+// prefix chosen so far; pass 0 also records the chunk's maximum.
+__global__ __launch_bounds__(SPL_THREADS) void split_hist_kernel(
+        const float* __restrict__ logits, size_t row_stride, int V, int pass, int with_hist,
+        SplitWs ws) {
+    __shared__ unsigned hist[256];
+    __shared__ float fscratch[16];
+    const int chunk = blockIdx.x, b = blockIdx.y;
+    float v[4];
+    int i0;
+    split_load(logits + b * row_stride, V, chunk, v, i0);
+    if (pass == 0) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (v[c] == v[c]) m = fmaxf(m, v[c]);
+        m = block_max(m, fscratch);
+        if (threadIdx.x == 0) ws.pmax[b * ws.NB + chunk] = m;
+    }
+    if (!with_hist) return;
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    const int shift = 24 - 8 * pass;
+    const uint32_t mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+    const uint32_t prefix = pass == 0 ? 0u : ws.state[b * 2];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        if (v[c] != v[c]) continue;
+        const uint32_t key = order_key(v[c]);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 256; i += blockDim.x)
+        if (hist[i]) atomicAdd(&ws.hist[(b * 4 + pass) * 256 + i], hist[i]);
+}
+
+// after a histogram pass: the bin that holds the k-th largest key extends the prefix.
+__global__ __launch_bounds__(256) void split_pick_kernel(int pass, int top_k, SplitWs ws) {
+    __shared__ unsigned suffix[257];
+    const int b = blockIdx.x, t = threadIdx.x;
+    suffix[t] = ws.hist[(b * 4 + pass) * 256 + t];
+    if (t == 0) suffix[256] = 0;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {          // suffix sums: suffix[t] = sum of bins >= t
+        const unsigned add = (t + off < 256) ? suffix[t + off] : 0u;
+        __syncthreads();
+        suffix[t] += add;
+        __syncthreads();
+    }
+    const unsigned rem = pass == 0 ? (unsigned)top_k : ws.state[b * 2 + 1];
+    const unsigned prefix = pass == 0 ? 0u : ws.state[b * 2];
+    __syncthreads();
+    if (suffix[t] >= rem && suffix[t + 1] < rem) {     // exactly one bin
+        ws.state[b * 2] = prefix | ((unsigned)t << (24 - 8 * pass));
+        ws.state[b * 2 + 1] = rem - suffix[t + 1];
+    }
+}
+
+__device__ __forceinline__ float split_row_max(const SplitWs& ws, int b) {
+    float m = -INFINITY;
+    for (int c = 0; c < ws.NB; ++c) m = fmaxf(m, ws.pmax[b * ws.NB + c]);
+    return m;
+}
+
+// partial sums of exp(v / t - max) over the kept entries of each chunk
+__global__ __launch_bounds__(SPL_THREADS) void split_sum_kernel(
+        const float* __restrict__ logits, size_t row_stride, int V, float t, int use_pivot,
+        SplitWs ws) {
+    __shared__ float fscratch[16];
+    const int chunk = blockIdx.x, b = blockIdx.y;
+    float v[4];
+    int i0;
+    split_load(logits + b * row_stride, V, chunk, v, i0);
+    const uint32_t pivot = use_pivot ? ws.state[b * 2] : 0u;
+    const float m = split_row_max(ws, b) / t;
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        if (v[c] == v[c] && order_key(v[c]) >= pivot) sum += expf(v[c] / t - m);
+    sum = block_sum(sum, fscratch);
+    if (threadIdx.x == 0) ws.psum[b * ws.NB + chunk] = sum;
+}
+
+// probabilities, the exponential race, and each chunk's best candidate
+__global__ __launch_bounds__(SPL_THREADS) void split_race_kernel(
+        const float* __restrict__ logits, size_t row_stride, int V, float t, int use_pivot,
+        uint32_t seed_lo, uint32_t seed_hi, const int* __restrict__ row_keys,
+        const int* __restrict__ positions, int position_offset, float* __restrict__ probs_out,
+        SplitWs ws) {
+    __shared__ ArgBest scratch[16];
+    const int chunk = blockIdx.x, b = blockIdx.y;
+    float v[4];
+    int i0;
+    split_load(logits + b * row_stride, V, chunk, v, i0);
+    const uint32_t pivot = use_pivot ? ws.state[b * 2] : 0u;
+    const float m = split_row_max(ws, b) / t;
+    float total = 0.f;
+    for (int c = 0; c < ws.NB; ++c) total += ws.psum[b * ws.NB + c];
+    uint32_t ctr[4] = {(uint32_t)(i0 >> 2), (uint32_t)(positions ? positions[b] + position_offset
+                                                                 : position_offset),
+                       (uint32_t)row_keys[b], 0u};
+    philox(ctr, seed_lo, seed_hi);
+    ArgBest best = {0.f, -1};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        if (i0 + c >= V) break;
+        float p = 0.f;
+        if (v[c] == v[c] && order_key(v[c]) >= pivot) p = expf(v[c] / t - m) / total;
+        if (probs_out) probs_out[(size_t)b * V + i0 + c] = p;
+        if (p > 0.f) {
+            ArgBest cand = {p / exp_noise(ctr[c]), i0 + c};
+            best = better(best, cand);
+        }
+    }
+    best = block_best(best, scratch);
+    if (threadIdx.x == 0) {
+        ws.pbest_v[b * ws.NB + chunk] = best.v;
+        ws.pbest_i[b * ws.NB + chunk] = best.i;
+    }
+}
+
+// each chunk's largest logit (greedy)
+__global__ __launch_bounds__(SPL_THREADS) void split_argmax_kernel(
+        const float* __restrict__ logits, size_t row_stride, int V, SplitWs ws) {
+    __shared__ ArgBest scratch[16];
+    const int chunk = blockIdx.x, b = blockIdx.y;
+    float v[4];
+    int i0;
+    split_load(logits + b * row_stride, V, chunk, v, i0);
+    ArgBest best = {0.f, -1};
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        if (v[c] == v[c]) {
+            ArgBest cand = {v[c], i0 + c};
+            best = better(best, cand);
+        }
+    best = block_best(best, scratch);
+    if (threadIdx.x == 0) {
+        ws.pbest_v[b * ws.NB + chunk] = best.v;
+        ws.pbest_i[b * ws.NB + chunk] = best.i;
+    }
+}
+
+__global__ __launch_bounds__(64) void split_final_kernel(int* __restrict__ out, SplitWs ws) {
+    const int b = blockIdx.x;
+    ArgBest best = {0.f, -1};
+    for (int c = threadIdx.x; c < ws.NB; c += 64) {
+        ArgBest cand = {ws.pbest_v[b * ws.NB + c], ws.pbest_i[b * ws.NB + c]};
+        best = better(best, cand);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgBest y;
+        y.v = __shfl_xor(best.v, o, 64);
+        y.i = __shfl_xor(best.i, o, 64);
+        best = better(best, y);
+    }
+    if (threadIdx.x == 0) out[b] = best.i < 0 ? 0 : best.i;
+}
+
+extern "C" size_t gfa_sample_split_workspace(int n_rows, int V) {
+    const size_t nb = (V + SPL_CHUNK - 1) / SPL_CHUNK;
+    return (size_t)n_rows * (4 * 256 + 2 + 4 * nb) * 4;
+}
+
+// temperature <= 0 means greedy.  `workspace` has gfa_sample_split_workspace bytes; its
+// first n_rows * 1024 ints (the histograms) must be zero at the call.
+extern "C" int gfa_sample_split(const float* logits, size_t row_stride, int n_rows, int V,
+                                float temperature, int top_k, uint64_t seed, const int* row_keys,
+                                const int* positions, int position_offset, int* out,
+                                float* probs_out, void* workspace, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    SplitWs ws;
+    ws.NB = (V + SPL_CHUNK - 1) / SPL_CHUNK;
+    char* p = (char*)workspace;
+    ws.hist = (unsigned*)p;      p += (size_t)n_rows * 4 * 256 * 4;
+    ws.state = (unsigned*)p;     p += (size_t)n_rows * 2 * 4;
+    ws.pmax = (float*)p;         p += (size_t)n_rows * ws.NB * 4;
+    ws.psum = (float*)p;         p += (size_t)n_rows * ws.NB * 4;
+    ws.pbest_v = (float*)p;      p += (size_t)n_rows * ws.NB * 4;
+    ws.pbest_i = (int*)p;
+    const dim3 grid(ws.NB, n_rows);
+    if (temperature <= 0.f) {
+        split_argmax_kernel<<<grid, SPL_THREADS, 0, stream>>>(logits, row_stride, V, ws);
+        split_final_kernel<<<n_rows, 64, 0, stream>>>(out, ws);
+        return GFA_LAUNCH_RESULT();
+    }
+    const float t = fmaxf(temperature, 1e-5f);
+    const int use_pivot = (top_k > 0 && top_k < V) ? 1 : 0;
+    for (int pass = 0; pass < (use_pivot ? 4 : 1); ++pass) {
+        split_hist_kernel<<<grid, SPL_THREADS, 0, stream>>>(logits, row_stride, V, pass, use_pivot, ws);
+        if (use_pivot) split_pick_kernel<<<n_rows, 256, 0, stream>>>(pass, top_k, ws);
+    }
+    split_sum_kernel<<<grid, SPL_THREADS, 0, stream>>>(logits, row_stride, V, t, use_pivot, ws);
+    split_race_kernel<<<grid, SPL_THREADS, 0, stream>>>(
+        logits, row_stride, V, t, use_pivot, (uint32_t)(seed & 0xffffffffu), (uint32_t)(seed >> 32),
+        row_keys, positions, position_offset, probs_out, ws);
+    split_final_kernel<<<n_rows, 64, 0, stream>>>(out, ws);
+    return GFA_LAUNCH_RESULT();
+}

@@ -222,6 +222,28 @@ def add_into(residual: torch.Tensor, y: torch.Tensor):
 
 
 # ----------------------------------------------------------------------------- sampling
+# vocabularies beyond this are spread over many workgroups per row
+SPLIT_SAMPLING_ABOVE = 16384
+
+
+def _split_workspace(B: int, V: int, device) -> torch.Tensor:
+    lib = library("sampling")
+    lib.gfa_sample_split_workspace.restype = ctypes.c_size_t
+    n = lib.gfa_sample_split_workspace(_i(B), _i(V))
+    return torch.zeros(n // 4, dtype=torch.int32, device=device)      # histograms start at zero
+
+
+def _sample_split(logits, temperature, top_k, seed, row_keys, positions, position_offset, out,
+                  probs):
+    B, V = logits.shape
+    ws = _split_workspace(B, V, logits.device)
+    check(library("sampling").gfa_sample_split(
+        ptr(logits), _sz(logits.stride(0)), _i(B), _i(V), _f(temperature), _i(top_k),
+        ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(row_keys), ptr(positions), _i(position_offset),
+        ptr(out), ptr(probs), ptr(ws), stream_handle()), "sample_split")
+    return out
+
+
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None):
     """int32 [B]: index of the largest of each row of float32 logits [B, V]."""
     require_device(logits)
@@ -231,6 +253,8 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None):
     B, V = logits.shape
     if out is None:
         out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    if V > SPLIT_SAMPLING_ABOVE:
+        return _sample_split(logits, 0.0, 0, 0, None, None, 0, out, None)
     check(library("sampling").gfa_argmax(ptr(logits), ptr(out), _i(B), _i(V),
                                          _sz(logits.stride(0)), stream_handle()), "argmax")
     return out
@@ -258,6 +282,11 @@ def sample(logits: torch.Tensor, temperature: float, top_k: Optional[int], seed:
     k = 0 if top_k is None else int(top_k)
     if k < 0:
         raise KernelError("sample: top_k must be positive")
+    if V > SPLIT_SAMPLING_ABOVE:
+        if temperature <= 0:
+            raise KernelError("sample: temperature must be positive (greedy is argmax)")
+        return _sample_split(logits, temperature, k, seed, row_keys, positions, position_offset,
+                             out, probs)
     check(library("sampling").gfa_sample(
         ptr(logits), _sz(logits.stride(0)), _i(B), _i(V), _f(temperature), _i(k),
         ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(row_keys), ptr(positions),

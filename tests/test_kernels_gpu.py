@@ -359,3 +359,36 @@ def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     close(q4, q2, 1e-2)
     close(kp4, kp2, 1e-2)
     assert torch.equal(vp4, vp2)                       # values are not rotated: same products
+
+
+def test_sampling_over_many_workgroups_equals_one_workgroup():
+    """Large vocabularies are spread over many workgroups per row; the choice, the
+    probabilities and the draws must be those of the one-workgroup kernels."""
+    from gpt_fast_amd.ops import kernels as KK
+    from gpt_fast_amd.sampling import SamplingParams, logits_to_probs, sample
+    torch.manual_seed(10)
+    B, V = 6, 50001                                     # no multiple of the chunk or of 4
+    logits = torch.randn(B, V, device=DEV) * 3
+    logits[1, 40000] = logits[1, 123] = 30.0            # a tie across chunks: lowest index
+    logits[2, 7] = float("nan")
+    keys = torch.arange(B, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([3, 1, 4, 1, 5, 9], dtype=torch.int32, device=DEV)
+    results = {}
+    for limit in (10 ** 9, 1000):                       # one workgroup per row / split
+        KK.SPLIT_SAMPLING_ABOVE = limit
+        try:
+            r = [KK.argmax(logits).cpu()]
+            for T, k in ((0.8, 200), (1.0, None), (0.5, 1), (1.3, 5000)):
+                r.append(sample(logits, SamplingParams(T, k, 11), keys, pos, 1).cpu())
+                r.append(logits_to_probs(logits, T, k).cpu())
+            results[limit] = r
+        finally:
+            KK.SPLIT_SAMPLING_ABOVE = 16384
+    one, split = results[10 ** 9], results[1000]
+    assert int(one[0][1]) == 123 and torch.equal(one[0], split[0])
+    for a, b in zip(one[1:], split[1:]):
+        if a.dtype == torch.int32:
+            assert torch.equal(a, b)
+        else:
+            assert torch.allclose(a, b, rtol=1e-5, atol=1e-9)
+            assert torch.equal(a > 0, b > 0)            # the same entries are kept

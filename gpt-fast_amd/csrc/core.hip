@@ -191,61 +191,53 @@ extern "C" int gfa_gemm_f32(const float* a, const float* w, float* out, int M, i
 // to page table[seq(n)][pos / PAGE], offset pos % PAGE (model.py:91-100, 206-207); keys as
 // rows [offset, hd], values transposed [hd, offset] (see common.h).
 template <typename T>
-__global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
-                                  T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                  const float* __restrict__ freqs,
-                                  const int* __restrict__ tok_seq,
-                                  const int* __restrict__ tok_pos,
-                                  const int* __restrict__ table, int table_stride, int H,
-                                  int Hkv, int hd, int rot, int layout) {
+__global__ __launch_bounds__(256) void rope_cache_kernel(
+        const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pages,
+        T* __restrict__ v_pages, const float* __restrict__ freqs, const int* __restrict__ tok_seq,
+        const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride, int H,
+        int Hkv, int hd, int rot, int layout) {
+    // one thread per pair of elements: q and k heads first (rotated or passed through), then
+    // the pairs of v; blockIdx.y walks the token's pairs in groups of 256
     const int n = blockIdx.x;
+    const int half = hd / 2;
+    const int rot_pairs = rot / 2;
+    const int qk_slots = (H + Hkv) * half, v_slots = Hkv * half;
+    const int e = blockIdx.y * 256 + threadIdx.x;
+    if (e >= qk_slots + v_slots) return;
     const int pos = tok_pos[n];
     const T* row = qkv + (size_t)n * (H + 2 * Hkv) * hd;
-    const int half = hd / 2;          // pairs per head when every element had a partner
-    const int rot_pairs = rot / 2;
-    size_t kv_base = 0;
-    int v_page = 0;
-    if (k_pages) {
-        v_page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
-        kv_base = page_row(v_page, 0, pos % GFA_PAGE, Hkv, hd);
-    }
-    // cos and sin of this token's angles, once for all heads
-    extern __shared__ float cs[];                  // [rot_pairs][2]
-    for (int i = threadIdx.x; i < rot_pairs; i += blockDim.x)
-        sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
-    __syncthreads();
-    // q and k heads: one thread per (head, pair-or-passthrough slot)
-    const int n_rot_heads = H + Hkv;
-    for (int e = threadIdx.x; e < n_rot_heads * half; e += blockDim.x) {
-        const int head = e / half, i = e % half;
+    int page = 0;
+    if (k_pages) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+    const int off = pos % GFA_PAGE;
+    if (e < qk_slots) {
+        const int head = e / half, i = e - head * half;
         const T* src = row + (size_t)head * hd;
         T* dst;
         if (head < H) {
             dst = q_out + ((size_t)n * H + head) * hd;
         } else {
-            if (!k_pages) continue;
-            dst = k_pages + kv_base + (size_t)(head - H) * GFA_PAGE * hd;
+            if (!k_pages) return;
+            dst = k_pages + page_row(page, head - H, off, Hkv, hd);
         }
         if (i < rot_pairs) {
             const int ia = layout == 0 ? 2 * i : i;
             const int ib = layout == 0 ? 2 * i + 1 : i + rot_pairs;
             const float a = load_as_float(src + ia), b = load_as_float(src + ib);
-            const float c = cs[2 * i], s = cs[2 * i + 1];
+            float s, c;
+            sincosf((float)pos * freqs[i], &s, &c);
             store_from_float(dst + ia, a * c - b * s);
             store_from_float(dst + ib, b * c + a * s);
         } else {
-            // elements rot .. hd-1 are copied, two per slot
-            const int d0 = rot + 2 * (i - rot_pairs);
+            const int d0 = rot + 2 * (i - rot_pairs);      // elements rot .. hd-1 are copied
             dst[d0] = src[d0];
             dst[d0 + 1] = src[d0 + 1];
         }
-    }
-    if (v_pages) {
-        const T* vsrc = row + (size_t)(H + Hkv) * hd;
-        for (int e = threadIdx.x; e < Hkv * hd; e += blockDim.x) {
-            const int g = e / hd, d = e % hd;
-            v_pages[value_elem(v_page, g, d, pos % GFA_PAGE, Hkv, hd)] = vsrc[e];
-        }
+    } else if (v_pages) {
+        const int ev = e - qk_slots;
+        const int g = ev / half, d = 2 * (ev - g * half);
+        const T* vsrc = row + (size_t)(H + Hkv + g) * hd + d;
+        v_pages[value_elem(page, g, d, off, Hkv, hd)] = vsrc[0];
+        v_pages[value_elem(page, g, d + 1, off, Hkv, hd)] = vsrc[1];
     }
 }
 
@@ -255,12 +247,13 @@ extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages,
                                     int Hkv, int hd, int rot, int layout, int is_bf16,
                                     hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    const dim3 grid(n_tokens, ((H + 2 * Hkv) * (hd / 2) + 255) / 256);
     if (is_bf16)
-        rope_cache_kernel<bf16_t><<<n_tokens, 256, (size_t)rot * sizeof(float), stream>>>(
+        rope_cache_kernel<bf16_t><<<grid, 256, 0, stream>>>(
             (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs,
             tok_seq, tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     else
-        rope_cache_kernel<float><<<n_tokens, 256, (size_t)rot * sizeof(float), stream>>>(
+        rope_cache_kernel<float><<<grid, 256, 0, stream>>>(
             (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, freqs, tok_seq,
             tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     return GFA_LAUNCH_RESULT();
@@ -373,10 +366,37 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
     }
 }
 
+// bfloat16 rows whose width is a multiple of 8: eight elements per thread, 16-byte accesses
+__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu,
+                                                              bf16_t* __restrict__ out, int I8,
+                                                              size_t total8) {
+    const size_t e = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (e >= total8) return;
+    const size_t n = e / I8;
+    const int i = (int)(e - n * I8);
+    const uint4 a = ((const uint4*)gu)[n * 2 * I8 + i], b = ((const uint4*)gu)[n * 2 * I8 + I8 + i];
+    const bf16_t* ae = (const bf16_t*)&a;
+    const bf16_t* be = (const bf16_t*)&b;
+    uint4 o;
+    bf16_t* oe = (bf16_t*)&o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float x = bf16_to_float(ae[j]);
+        oe[j] = float_to_bf16((x / (1.f + expf(-x))) * bf16_to_float(be[j]));
+    }
+    ((uint4*)out)[e] = o;
+}
+
 extern "C" int gfa_silu_mul(const void* gu, void* out, int n_rows, int I, int is_bf16,
                             hipStream_t stream) {
     const size_t total = (size_t)n_rows * I;
     if (total == 0) return 0;
+    if (is_bf16 && I % 8 == 0) {
+        const size_t total8 = total / 8;
+        silu_mul_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
+            (const bf16_t*)gu, (bf16_t*)out, I / 8, total8);
+        return GFA_LAUNCH_RESULT();
+    }
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     if (is_bf16)
         silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
@@ -394,9 +414,30 @@ __global__ void add_into_kernel(float* __restrict__ res, const T* __restrict__ y
         res[e] += load_as_float(y + e);
 }
 
+// bfloat16 addend, four elements per thread
+__global__ __launch_bounds__(256) void add_into_bf16x4_kernel(float4* __restrict__ res,
+                                                              const uint2* __restrict__ y,
+                                                              size_t total4) {
+    const size_t e = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (e >= total4) return;
+    float4 r = res[e];
+    const uint2 v = y[e];
+    r.x += __uint_as_float(v.x << 16);
+    r.y += __uint_as_float(v.x & 0xffff0000u);
+    r.z += __uint_as_float(v.y << 16);
+    r.w += __uint_as_float(v.y & 0xffff0000u);
+    res[e] = r;
+}
+
 extern "C" int gfa_add_into(float* res, const void* y, size_t total, int y_bf16,
                             hipStream_t stream) {
     if (total == 0) return 0;
+    if (y_bf16 && total % 4 == 0 && ((uintptr_t)res % 16 == 0) && ((uintptr_t)y % 8 == 0)) {
+        const size_t total4 = total / 4;
+        add_into_bf16x4_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, stream>>>(
+            (float4*)res, (const uint2*)y, total4);
+        return GFA_LAUNCH_RESULT();
+    }
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     if (y_bf16)
         add_into_kernel<bf16_t><<<blocks, 256, 0, stream>>>(res, (const bf16_t*)y, total);

@@ -278,6 +278,279 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     }
 }
 
+// --------------------------------------------------------------------------------------
+// Prompts: a workgroup of four waves owns 128 query rows (32 per wave) of one sequence and
+// kv head and walks the keys a page (64 keys) at a time.  The page's keys and values are
+// copied once into LDS by all four waves - each is one contiguous piece of the cache - and
+// the next page is already on its way while the current one is multiplied.  Rows of the
+// LDS tiles are padded so that the operand reads (16 rows at a time) spread over the banks.
+// The arithmetic per 32 keys is that of the kernel above.
+#define TL_WAVES 4
+#define TL_RT 2
+#define TL_ROWS (TL_WAVES * TL_RT * 16)
+
+template <int DS>
+__global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
+        const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+        const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
+        const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
+        bf16_t* __restrict__ out, int H, int Hkv, int hd, float scale_log2, int window) {
+    constexpr int DT = DS * 2, RT = TL_RT;
+    constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
+    constexpr int KPITCH = HDM * 2 + 16;                  // bytes per key row in LDS
+    constexpr int VPITCH = 64 * 2 + 8;                    // bytes per value row (one dim, 64 keys)
+    constexpr int KBYTES = 64 * KPITCH, VBYTES = HDM * VPITCH;
+    extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 x (K tile, V tile)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int g = blockIdx.y, seq = blockIdx.z;
+    const int R = H / Hkv;
+    const int q0 = q_start[seq];
+    const int rows_total = (q_start[seq + 1] - q0) * R;
+    // later tiles see more keys: hand them out first so that the longest work starts first
+    const int wg_row0 = (gridDim.x - 1 - blockIdx.x) * TL_ROWS;
+    if (wg_row0 >= rows_total) return;
+    const int spos = start_pos[seq];
+    const int* pages = table + (size_t)seq * table_stride;
+    const int row0 = wg_row0 + wave * RT * 16;            // this wave's first row (may be beyond the end)
+
+    Frag qf[RT][DS];
+    int rpos[RT];
+    size_t orow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int r = row0 + rt * 16 + li;
+        const bool valid = r < rows_total;
+        const int t = valid ? r / R : 0, hh = valid ? r - (r / R) * R : 0;
+        rpos[rt] = valid ? spos + t : -1;
+        orow[rt] = (size_t)(q0 + t) * H + g * R + hh;
+        const bf16_t* qrow = q + orow[rt] * hd;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int d = ds * 32 + lg * 8;
+            qf[rt][ds].u = (valid && d < hd) ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
+        }
+    }
+    // key range of the workgroup and of this wave
+    const int wg_last = (wg_row0 + TL_ROWS - 1 < rows_total - 1) ? wg_row0 + TL_ROWS - 1 : rows_total - 1;
+    const int wg_pmin = spos + wg_row0 / R, wg_pmax = spos + wg_last / R;
+    const bool wave_has_rows = row0 < rows_total;
+    const int w_last = (row0 + RT * 16 - 1 < rows_total - 1) ? row0 + RT * 16 - 1 : rows_total - 1;
+    const int pmin = wave_has_rows ? spos + row0 / R : 0;
+    const int pmax = wave_has_rows ? spos + w_last / R : -1;
+    const int lo = (window > 0 && wg_pmin - window + 1 > 0) ? wg_pmin - window + 1 : 0;
+    const int w_lo = (window > 0 && pmin - window + 1 > 0) ? pmin - window + 1 : 0;
+    const int page_lo = lo >> 6, page_hi = wg_pmax >> 6;
+
+    float m[RT], l[RT];
+    floatx4_t o[RT][DT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // staging: a page's keys are 64 * hd * 2 contiguous bytes, its values hd * 64 * 2
+    const int k_chunks = 64 * hd / 8, v_chunks = hd * 64 / 8;      // 16-byte pieces
+    constexpr int K_PER = (64 * HDM / 8 + 255) / 256, V_PER = (HDM * 64 / 8 + 255) / 256;
+    uint4 kreg[K_PER], vreg[V_PER];
+    auto fetch_page = [&](int pg) {
+        const int page = pages[pg];
+        const uint4* ksrc = (const uint4*)(k_pages + page_row(page, g, 0, Hkv, hd));
+        const uint4* vsrc = (const uint4*)(v_pages + value_elem(page, g, 0, 0, Hkv, hd));
+#pragma unroll
+        for (int i = 0; i < K_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            kreg[i] = c < k_chunks ? ksrc[c] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            vreg[i] = c < v_chunks ? vsrc[c] : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto store_page = [&](int buf, int pg) {
+        char* kt = smem + buf * (KBYTES + VBYTES);
+        char* vt = kt + KBYTES;
+        const int hd8 = hd / 8;                            // 16-byte pieces per key row
+        const int keys_ok = wg_pmax - pg * 64;             // keys beyond hold no data yet
+#pragma unroll
+        for (int i = 0; i < K_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < k_chunks) {
+                const int key = c / hd8, piece = c - key * hd8;
+                *(uint4*)(kt + key * KPITCH + piece * 16) = kreg[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < v_chunks) {
+                const int d = c >> 3, piece = c & 7;       // 8 pieces of 8 keys per dim
+                Frag f;
+                f.u = vreg[i];
+                if (piece * 8 + 7 > keys_ok) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (piece * 8 + e > keys_ok) f.e[e] = 0;
+                }
+                uint2* dst = (uint2*)(vt + d * VPITCH + piece * 16);
+                dst[0] = f.h[0];
+                dst[1] = f.h[1];
+            }
+        }
+    };
+    auto compute_block = [&](int buf, int kb) {            // kb: block of 32 keys
+        const char* kt = smem + buf * (KBYTES + VBYTES);
+        const char* vt = kt + KBYTES;
+        const int in_page = (kb & 1) * 32;
+        const int key0 = kb * 32 + lg * 4;
+        floatx4_t s[RT][2];
+#pragma unroll
+        for (int kt16 = 0; kt16 < 2; ++kt16) {
+            Frag kf[DS];
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds)
+                kf[ds].u = (ds * 32 + lg * 8 < hd)
+                               ? *(const uint4*)(kt + (in_page + kt16 * 16 + li) * KPITCH + (ds * 32 + lg * 8) * 2)
+                               : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                s[rt][kt16] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < DS; ++ds)
+                    s[rt][kt16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ds].v, qf[rt][ds].v, s[rt][kt16], 0, 0, 0);
+            }
+        }
+        const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
+        Frag pf[RT];
+        float alpha[RT];
+        bool rescale = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            float sv[8];
+            float mx = -INFINITY;
+            if (masked) {
+                const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int key = key0 + (e >> 2) * 16 + (e & 3);
+                    const float v = s[rt][e >> 2][e & 3] * scale_log2;
+                    sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
+                    mx = fmaxf(mx, sv[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    sv[e] = s[rt][e >> 2][e & 3] * scale_log2;
+                    mx = fmaxf(mx, sv[e]);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m[rt], mx);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - m_safe);
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = __builtin_amdgcn_exp2f(sv[e] - m_safe);
+                sum += p;
+                pf[rt].e[e] = float_to_bf16(p);
+            }
+            l[rt] = l[rt] * alpha[rt] + sum;
+            m[rt] = m_new;
+            rescale = rescale || (__builtin_amdgcn_ballot_w64(alpha[rt] != 1.f) != 0);
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            if (dt * 16 < hd) {
+                Frag vf;
+                const char* vrow = vt + (dt * 16 + li) * VPITCH + (in_page + lg * 4) * 2;
+                vf.h[0] = *(const uint2*)vrow;
+                vf.h[1] = *(const uint2*)(vrow + 32);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    if (rescale) o[rt][dt] *= alpha[rt];
+                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][dt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    fetch_page(page_lo);
+    store_page(0, page_lo);
+    __syncthreads();
+    for (int pg = page_lo; pg <= page_hi; ++pg) {
+        const int buf = (pg - page_lo) & 1;
+        if (pg < page_hi) fetch_page(pg + 1);
+        if (wave_has_rows) {
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {
+                const int kb = pg * 2 + hb;
+                if (kb * 32 <= pmax && kb * 32 + 31 >= w_lo) compute_block(buf, kb);
+            }
+        }
+        if (pg < page_hi) store_page(buf ^ 1, pg + 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float lt = l[rt] + __shfl_xor(l[rt], 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (rpos[rt] < 0) continue;
+        const float inv = 1.f / lt;
+        bf16_t* orow_p = out + orow[rt] * hd;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int d = dt * 16 + lg * 4;
+            if (d < hd) {
+                Frag w;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w.e[j] = float_to_bf16(o[rt][dt][j] * inv);
+                *(uint2*)(orow_p + d) = w.h[0];
+            }
+        }
+    }
+}
+
+template <int DS>
+static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k,
+                                   const bf16_t* v, const int* q_start, const int* start_pos,
+                                   const int* table, int table_stride, bf16_t* out, int H, int Hkv,
+                                   int hd, float sl2, int window) {
+    constexpr int HDM = DS * 32;
+    const size_t shmem = 2 * (size_t)(64 * (HDM * 2 + 16) + HDM * (64 * 2 + 8));
+    static bool raised = false;
+    if (!raised) {
+        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        raised = true;
+    }
+    attention_tiled_kernel<DS><<<grid, 256, shmem, stream>>>(q, k, v, q_start, start_pos, table,
+                                                             table_stride, out, H, Hkv, hd, sl2, window);
+}
+
+// Prompts of many rows: max_tiles = most 128-row tiles any sequence needs per kv head.
+extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, const void* v_pages,
+                                        const int* q_start, const int* start_pos, const int* table,
+                                        int table_stride, void* out, int n_tokens, int n_seqs, int H,
+                                        int Hkv, int hd, float scale, int window, int max_tiles,
+                                        hipStream_t stream) {
+    if (n_tokens <= 0 || n_seqs <= 0) return 0;
+    if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_tiles < 1) return (int)hipErrorInvalidValue;
+    const dim3 grid(max_tiles, Hkv, n_seqs);
+    const float sl2 = scale * LOG2E;
+    if (hd <= 64)
+        launch_attention_tiled<2>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    else
+        launch_attention_tiled<4>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    return GFA_LAUNCH_RESULT();
+}
+
 // out[row, :] = sum_s w_s o_s / sum_s w_s l_s with w_s = 2^(m_s - max m), splits in order.
 __global__ void attention_combine_kernel(const float* __restrict__ ws_o,
                                          const float* __restrict__ ws_ml, bf16_t* __restrict__ out,

@@ -13,6 +13,8 @@ MIN_KEYS_PER_SPLIT = 128
 MAX_SPLITS = 16
 
 
+TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
+                           # the workgroup-tiled kernel (keys and values through LDS)
 PREFILL_ROW_TILES = 4      # 16-row tiles per wave for prompts
 
 
@@ -53,6 +55,15 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
     if batch.q_start.numel() != batch.n_seqs + 1 or batch.start_pos.numel() != batch.n_seqs \
             or table.shape[0] != batch.n_seqs or table.dtype != torch.int32:
         raise KernelError("attention_bf16: the batch description does not fit its sequences")
+    R = H // G
+    if batch.max_q_len * R >= TILED_MIN_ROWS and hd <= 128:
+        out = torch.empty_like(q)
+        tiles = (batch.max_q_len * R + 127) // 128
+        check(library("attention_bf16").gfa_attention_tiled_bf16(
+            ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos),
+            ptr(table), _i(table.shape[1]), ptr(out), _i(n), _i(batch.n_seqs), _i(H), _i(G), _i(hd),
+            _f(scale), _i(window), _i(tiles), stream_handle()), "attention_tiled_bf16")
+        return out
     rt, nw, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
     out = torch.empty_like(q)
     ws_o = ws_ml = None

@@ -202,9 +202,16 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
     const int half = hd / 2;
     const int rot_pairs = rot / 2;
     const int qk_slots = (H + Hkv) * half, v_slots = Hkv * half;
+    const int pos = tok_pos[n];
+    // cos and sin of this token's angles, once per workgroup
+    extern __shared__ float cs[];                          // [rot_pairs][2]
+    if (blockIdx.y * 256 < qk_slots) {
+        for (int i = threadIdx.x; i < rot_pairs; i += 256)
+            sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
+        __syncthreads();
+    }
     const int e = blockIdx.y * 256 + threadIdx.x;
     if (e >= qk_slots + v_slots) return;
-    const int pos = tok_pos[n];
     const T* row = qkv + (size_t)n * (H + 2 * Hkv) * hd;
     int page = 0;
     if (k_pages) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
@@ -223,8 +230,7 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
             const int ia = layout == 0 ? 2 * i : i;
             const int ib = layout == 0 ? 2 * i + 1 : i + rot_pairs;
             const float a = load_as_float(src + ia), b = load_as_float(src + ib);
-            float s, c;
-            sincosf((float)pos * freqs[i], &s, &c);
+            const float c = cs[2 * i], s = cs[2 * i + 1];
             store_from_float(dst + ia, a * c - b * s);
             store_from_float(dst + ib, b * c + a * s);
         } else {
@@ -249,11 +255,11 @@ extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages,
     if (n_tokens <= 0) return 0;
     const dim3 grid(n_tokens, ((H + 2 * Hkv) * (hd / 2) + 255) / 256);
     if (is_bf16)
-        rope_cache_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        rope_cache_kernel<bf16_t><<<grid, 256, (size_t)rot * sizeof(float), stream>>>(
             (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs,
             tok_seq, tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     else
-        rope_cache_kernel<float><<<grid, 256, 0, stream>>>(
+        rope_cache_kernel<float><<<grid, 256, (size_t)rot * sizeof(float), stream>>>(
             (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, freqs, tok_seq,
             tok_pos, table, table_stride, H, Hkv, hd, rot, layout);
     return GFA_LAUNCH_RESULT();

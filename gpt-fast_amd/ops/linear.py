@@ -4,9 +4,9 @@ reference's linears (model.py:110, 174-175, 222-224), with the epilogues the blo
 float32 engine: the library's own float32 kernel, for every shape (a true 32-bit
 product; one fused-multiply-add chain per output).
 
-bfloat16 engine: hand-written kernels for the few-row products of decoding (weights are
-streamed once; see csrc/gemm_bf16.hip); the vendor matrix library, through
-``torch.matmul``, for the many-row products of prefill - the reference uses the vendor
+bfloat16 engine: hand-written kernels for the few-row products of decoding (up to 16
+rows; weights are streamed once; see csrc/gemm_bf16.hip); the vendor matrix library,
+through ``torch.matmul``, for products of more rows - the reference uses the vendor
 library for these as well.  Accumulation is float32 everywhere.
 """
 from typing import Optional

@@ -356,3 +356,83 @@ def test_graph_replays_equal_eager_steps_for_any_batch_size(tmp_path_factory, n_
         for s in slots:
             eng.end_sequence(s)
     assert runs[True] == runs[False]
+
+
+def _plain_forward_with_windows(w, cfg, tokens, windows):
+    """The plain model with a window per layer (None: all keys): the causal mask of
+    model.py:134 with keys at distance >= window masked as well."""
+    import math
+    idx = torch.as_tensor(tokens, dtype=torch.long)
+    S = idx.numel()
+    pos = torch.arange(S)
+    x = w["tok_embeddings.weight"][idx]
+    H, G, hd = cfg["n_head"], cfg["n_kv"], cfg["head_dim"]
+    for i, win in enumerate(windows):
+        p = f"layers.{i}."
+        xn = plain.rms_norm(x, w[p + "attention_norm.weight"], cfg["eps"])
+        qkv = xn @ w[p + "attention.wqkv.weight"].T
+        q, k, v = qkv.split([H * hd, G * hd, G * hd], dim=-1)
+        cos, sin = plain.rope_table(pos, hd, cfg["rope_base"], cfg["rope_scaling"])
+        q = plain.apply_rope(q.reshape(S, H, hd), cos, sin)
+        k = plain.apply_rope(k.reshape(S, G, hd), cos, sin)
+        v = v.reshape(S, G, hd)
+        keep = torch.tril(torch.ones(S, S, dtype=torch.bool))
+        if win is not None:
+            keep &= (pos[:, None] - pos[None, :]) < win
+        y = torch.empty(S, H, hd)
+        for h in range(H):
+            g = h // (H // G)
+            s = (q[:, h] @ k[:, g].T) / math.sqrt(hd)
+            y[:, h] = torch.softmax(s.masked_fill(~keep, float("-inf")), -1) @ v[:, g]
+        x = x + y.reshape(S, H * hd) @ w[p + "attention.wo.weight"].T
+        x = x + plain.feed_forward(plain.rms_norm(x, w[p + "ffn_norm.weight"], cfg["eps"]),
+                                   w[p + "feed_forward.w1.weight"], w[p + "feed_forward.w3.weight"],
+                                   w[p + "feed_forward.w2.weight"])
+    return plain.rms_norm(x, w["norm.weight"], cfg["eps"]) @ w["output.weight"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32), ("bfloat16", TOL_BF16)])
+def test_layers_with_windows_have_storage_of_their_own(tmp_path_factory, dtype, tol):
+    """A plan (made here, not an architecture of the library) whose layers differ: full
+    attention, a window of 70 keys, a window of 20.  Each need gets its own cache group;
+    the windowed groups give pages back while the sequence grows; logits equal the plain
+    model with the same windows, whole, cut into steps, and next to another sequence."""
+    import dataclasses
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.weights.bindings import load_parameters
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    arch, cfg = gfa.read_model_folder(folder)
+    plan = arch.plan(cfg)
+    windows = [None, 70, 20]
+    plan.layers = [dataclasses.replace(layer, mixer=dataclasses.replace(layer.mixer, window=win))
+                   for layer, win in zip(plan.layers, windows)]
+    params = load_parameters(folder, arch.bindings(cfg), dtype, torch.device("cuda:0"))
+    eng = gfa.Engine.from_plan(plan, params, dtype, "cuda:0", max_tokens=64 * 12)
+    assert len(eng.cache.kv_groups) == 3
+    pcfg, w = plain.load_folder(folder)
+    toks = util.random_tokens(pcfg["vocab"], 300, 9)
+    want = _plain_forward_with_windows(w, pcfg, toks, windows)
+    slot = eng.start_sequence()
+    whole = eng.step([Entry(slot, toks, want=list(range(300)))]).cpu()
+    assert rel_err(whole, want) < tol
+    held = [g.pages.held for _, g in eng.cache.kv_groups]
+    assert held == [5, 5, 5]                      # a whole prompt needs every page while it runs
+    eng.end_sequence(slot)
+    # prompt, then token by token, beside a second sequence: windowed groups let pages go
+    a, b = eng.start_sequence(), eng.start_sequence()
+    other = util.random_tokens(pcfg["vocab"], 80, 10)
+    got = [eng.step([Entry(a, toks[:150], want=list(range(150))), Entry(b, other[:40])]).cpu()]
+    for i in range(150, 300):
+        entries = [Entry(a, [toks[i]], want=[0])]
+        if i < 190:
+            entries.append(Entry(b, [other[i - 110]]))
+        got.append(eng.step(entries).cpu())
+    assert rel_err(torch.cat(got), want) < tol
+    held = {g.need.window: len([p for p in eng.cache.page_list(gid, a) if p >= 0])
+            for gid, g in eng.cache.kv_groups}
+    assert held[None] == 5 and held[70] == 2 and held[20] == 1
+    eng.cache.check()
+    eng.end_sequence(a)
+    eng.end_sequence(b)
+    assert all(g.pages.held == 0 for _, g in eng.cache.kv_groups)

@@ -138,8 +138,12 @@ def _attention_ref(q, k, v, pos, scale, window):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1.5e-2)])
-@pytest.mark.parametrize("H,G,hd,window", [(4, 4, 16, 0), (6, 2, 48, 0), (8, 1, 128, 0),
-                                           (3, 3, 80, 0), (4, 2, 64, 37), (2, 1, 256, 100)])
+@pytest.mark.parametrize("H,G,hd,window", [
+    (4, 4, 16, 0), (6, 2, 48, 0), (8, 1, 128, 0), (3, 3, 80, 0), (4, 2, 64, 37), (2, 1, 256, 100),
+    (32, 1, 64, 0),                 # 32 heads on one kv head: two row tiles per token
+    (7, 7, 32, 0), (10, 2, 112, 0), (9, 3, 96, 65), (5, 1, 144, 0), (2, 2, 176, 0), (3, 1, 208, 0),
+    (2, 1, 240, 0), (12, 4, 128, 33), (4, 1, 20, 0), (2, 2, 264, 0),      # last two: plain kernel only
+])
 def test_attention_over_pages(dtype, tol, H, G, hd, window):
     """Prefill rows (many tokens of a sequence) and decode rows (its last token) in one
     launch, sequences of unequal length on scattered pages, unused page tails poisoned."""

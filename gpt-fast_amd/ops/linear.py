@@ -61,27 +61,11 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
     return K.silu_mul(torch.matmul(x, w13.t()))
 
 
-# ----------------------------------------------------------------------------- fused with the norm
-def can_fuse_norm(residual: torch.Tensor, norm, w: torch.Tensor) -> bool:
-    """True if the few-row kernels can read ``residual`` through ``norm`` themselves: a
-    bfloat16 engine, an RMS norm, at most 64 rows, an inner size that is a multiple of 8."""
-    return (w.dtype == torch.bfloat16 and getattr(getattr(norm, "spec", None), "kind", None) == "rms"
-            and getattr(norm, "weight", None) is not None
-            and _fast().can_fuse_norm(residual.shape[0], w.shape[1]))
-
-
+# ----------------------------------------------------------------------------- fused projection
 def can_project_rotate_store(x: torch.Tensor, wqkv: torch.Tensor, head_dim: int) -> bool:
     """True if the fused projection / rotation / cache-write kernel takes these rows."""
     return (x.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
             and wqkv.shape[1] % 8 == 0 and head_dim % 16 == 0)
-
-
-def gated_linear_normed(residual, norm_w, eps, w13):
-    return _fast().skinny_normed_gated(residual, norm_w, eps, w13)
-
-
-def linear_normed(residual, norm_w, eps, w, out_dtype=torch.bfloat16):
-    return _fast().skinny_normed(residual, norm_w, eps, w, out_dtype=out_dtype)
 
 
 def qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,

@@ -37,14 +37,8 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     def forward(self, residual, batch, entry):
-        # a part may take the residual stream and its norm together (one fused kernel);
-        # it says so by returning True from forward_normed
-        fused = getattr(self.mixer, "forward_normed", None)
-        if fused is None or not fused(residual, self.mixer_norm, batch, entry):
-            self.mixer.forward(self.mixer_norm.forward(residual), batch, entry, residual)
-        fused = getattr(self.feed_forward, "forward_normed", None)
-        if fused is None or not fused(residual, self.feed_forward_norm, batch):
-            self.feed_forward.forward(self.feed_forward_norm.forward(residual), batch, residual)
+        self.mixer.forward(self.mixer_norm.forward(residual), batch, entry, residual)
+        self.feed_forward.forward(self.feed_forward_norm.forward(residual), batch, residual)
 
 
 register_block("pre_norm", PreNormBlock)

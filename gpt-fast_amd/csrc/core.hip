@@ -116,6 +116,93 @@ extern "C" int gfa_rmsnorm(const float* x, const float* w, const int* rows, void
 }
 
 // --------------------------------------------------------------------------------------
+// The sum that completes a block and the norm that opens the next, one pass over each row:
+// res[i, :] += float(y[i, :]);  out[i, :] = rmsnorm(res[i, :]) in bfloat16
+// (model.py:162-163 followed by 236-241; the sum and the statistics in float)
+__global__ void add_rmsnorm_kernel(float* __restrict__ res, const bf16_t* __restrict__ y,
+                                   const float* __restrict__ w, bf16_t* __restrict__ out, int dim,
+                                   float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    float* xr = res + (size_t)i * dim;
+    const bf16_t* yr = y + (size_t)i * dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        const float v = xr[d] + bf16_to_float(yr[d]);
+        xr[d] = v;                                       // read back by this thread only
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float rs = rsqrtf(ss / (float)dim + eps);
+    bf16_t* o = out + (size_t)i * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) store_from_float(o + d, xr[d] * rs * w[d]);
+}
+
+// rows of up to 1024 * VPT elements (a multiple of 4), kept in registers
+template <int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(
+        float* __restrict__ res, const bf16_t* __restrict__ y, const float* __restrict__ w,
+        bf16_t* __restrict__ out, int dim, float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    float4* xr = (float4*)(res + (size_t)i * dim);
+    const uint2* yr = (const uint2*)(y + (size_t)i * dim);
+    const float4* w4 = (const float4*)w;
+    const int n4 = dim >> 2;
+    float4 v[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (idx < n4) {
+            v[j] = xr[idx];
+            const uint2 a = yr[idx];
+            v[j].x += __uint_as_float(a.x << 16);
+            v[j].y += __uint_as_float(a.x & 0xffff0000u);
+            v[j].z += __uint_as_float(a.y << 16);
+            v[j].w += __uint_as_float(a.y & 0xffff0000u);
+            xr[idx] = v[j];
+        }
+        ss = fmaf(v[j].x, v[j].x, ss);
+        ss = fmaf(v[j].y, v[j].y, ss);
+        ss = fmaf(v[j].z, v[j].z, ss);
+        ss = fmaf(v[j].w, v[j].w, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float rs = rsqrtf(ss / (float)dim + eps);
+    uint2* o = (uint2*)(out + (size_t)i * dim);
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            const float4 g = w4[idx];
+            bf16_t e[4];
+            e[0] = float_to_bf16(v[j].x * rs * g.x);
+            e[1] = float_to_bf16(v[j].y * rs * g.y);
+            e[2] = float_to_bf16(v[j].z * rs * g.z);
+            e[3] = float_to_bf16(v[j].w * rs * g.w);
+            o[idx] = make_uint2((unsigned)e[0] | ((unsigned)e[1] << 16),
+                                (unsigned)e[2] | ((unsigned)e[3] << 16));
+        }
+    }
+}
+
+extern "C" int gfa_add_rmsnorm(float* res, const void* y, const float* w, void* out, int n_rows,
+                               int dim, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    const bf16_t* yp = (const bf16_t*)y;
+    bf16_t* op = (bf16_t*)out;
+    const bool vec = dim % 4 == 0 && dim <= 8192 && (uintptr_t)res % 16 == 0 &&
+                     (uintptr_t)y % 8 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)w % 16 == 0;
+    if (!vec) add_rmsnorm_kernel<<<n_rows, 256, 0, stream>>>(res, yp, w, op, dim, eps);
+    else if (dim <= 1024) add_rmsnorm_vec_kernel<1, 256><<<n_rows, 256, 0, stream>>>(res, yp, w, op, dim, eps);
+    else if (dim <= 4096) add_rmsnorm_vec_kernel<1, 1024><<<n_rows, 1024, 0, stream>>>(res, yp, w, op, dim, eps);
+    else add_rmsnorm_vec_kernel<2, 1024><<<n_rows, 1024, 0, stream>>>(res, yp, w, op, dim, eps);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
 // float32 matrix product: out[m, n] (+)= sum_k a[m, k] * w[n, k]
 // 64x64 tile per workgroup of 256 threads, 4x4 outputs per thread, k in steps of 16 through
 // shared memory.  Each output is one fused-multiply-add chain over k = 0..K-1 in order.

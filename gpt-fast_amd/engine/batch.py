@@ -85,6 +85,10 @@ class StepBatch:
         self.max_q_len = int(q_lens.max()) if self.n_seqs else 0
         self.max_kv_len = int((start + q_lens).max()) if self.n_seqs else 0
         self.is_decode = self.max_q_len == 1
+        w_off, _ = layout.fields["want_rows"]
+        # every row's logits are wanted, in order: the final norm needs no gather
+        self.every_row_wanted = self.n_want == self.n_tokens and bool(
+            (host[w_off:w_off + self.n_want] == np.arange(self.n_want)).all())
 
     def table(self, group_id: int) -> torch.Tensor:
         return self._tables[group_id]

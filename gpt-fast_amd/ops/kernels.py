@@ -221,6 +221,23 @@ def add_into(residual: torch.Tensor, y: torch.Tensor):
     return residual
 
 
+def add_rmsnorm(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float):
+    """residual += float(y), then the RMS norm of the new rows in bfloat16: one pass.
+    residual float32 [N, D], y bfloat16 [N, D], weight float32 [D]."""
+    require_device(residual, y, weight)
+    require_contiguous(residual=residual, y=y, weight=weight)
+    _want(residual, torch.float32, "residual")
+    _want(weight, torch.float32, "norm weight")
+    _want(y, torch.bfloat16, "y")
+    if residual.dim() != 2 or y.shape != residual.shape or weight.numel() != residual.shape[1]:
+        raise KernelError("add_rmsnorm: shapes of residual, y and the norm weight do not fit")
+    out = torch.empty(residual.shape, dtype=torch.bfloat16, device=residual.device)
+    check(library("core").gfa_add_rmsnorm(ptr(residual), ptr(y), ptr(weight), ptr(out),
+                                          _i(residual.shape[0]), _i(residual.shape[1]), _f(eps),
+                                          stream_handle()), "add_rmsnorm")
+    return out
+
+
 # ----------------------------------------------------------------------------- sampling
 # vocabularies beyond this are spread over many workgroups per row
 SPLIT_SAMPLING_ABOVE = 16384

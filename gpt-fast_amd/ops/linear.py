@@ -42,8 +42,20 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return torch.matmul(x, w.t())
 
 
-def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor):
-    """residual (float32 [M, N]) += x W^T."""
+def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_norm=None):
+    """residual (float32 [M, N]) += x W^T.  ``then_norm``: the norm that reads the residual
+    stream next.  Where the sum is a kernel of its own (many bfloat16 rows) and the norm is a
+    factor per row times a weight per column, sum and norm run as one pass and the normed
+    rows are returned; else None, and the caller runs the norm."""
+    form = getattr(then_norm, "row_and_column_form", None)
+    if form is not None and x.dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS:
+        weight, eps = form()
+        return K.add_rmsnorm(residual, torch.matmul(x, w.t()), weight, eps)
+    _linear_into(x, w, residual)
+    return None
+
+
+def _linear_into(x, w, residual):
     if x.dtype == torch.float32:
         return K.gemm_f32(x, w, out=residual, accumulate=True)
     if x.shape[0] <= SKINNY_MAX_ROWS:

@@ -39,7 +39,9 @@ class Attention(Part):
         s = self.spec
         return KVNeed(s.n_kv_heads, s.head_dim, s.window)
 
-    def forward(self, x, batch, entry, residual):
+    prepares_norm = True
+
+    def forward(self, x, batch, entry, residual, then_norm=None):
         s = self.spec
         q = None
         fused = getattr(self.position, "project_rotate_store", None)
@@ -52,7 +54,8 @@ class Attention(Part):
                                                s.head_dim)                  # model.py:201-207
         y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
                         self.scale, self.window)                            # model.py:209-211
-        L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual)  # :215, 162
+        return L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual,
+                             then_norm)                                     # model.py:215, 162
 
 
 register_mixer("attention", Attention)

@@ -36,9 +36,27 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, residual, batch, entry):
-        self.mixer.forward(self.mixer_norm.forward(residual), batch, entry, residual)
-        self.feed_forward.forward(self.feed_forward_norm.forward(residual), batch, residual)
+    # Norm hand-over, optional for every part: a mixer or feed-forward that sets
+    # ``prepares_norm`` takes ``then_norm=`` (the norm that reads the residual stream after
+    # it) and returns that norm's rows if it produced them on the way, else None.  A block
+    # that sets it takes ``x=`` (the rows of its first norm, if the caller has them) and
+    # ``then_norm=`` in the same sense, and names its first norm ``mixer_norm``.
+    prepares_norm = True
+
+    def forward(self, residual, batch, entry, x=None, then_norm=None):
+        if x is None:
+            x = self.mixer_norm.forward(residual)
+        h = None
+        if getattr(self.mixer, "prepares_norm", False):
+            h = self.mixer.forward(x, batch, entry, residual, then_norm=self.feed_forward_norm)
+        else:
+            self.mixer.forward(x, batch, entry, residual)
+        if h is None:
+            h = self.feed_forward_norm.forward(residual)
+        if then_norm is not None and getattr(self.feed_forward, "prepares_norm", False):
+            return self.feed_forward.forward(h, batch, residual, then_norm=then_norm)
+        self.feed_forward.forward(h, batch, residual)
+        return None
 
 
 register_block("pre_norm", PreNormBlock)

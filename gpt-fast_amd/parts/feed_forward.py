@@ -23,9 +23,11 @@ class GatedFeedForward(Part):
         check_bound("GatedFeedForward", self.parameters(), tensors)
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
-    def forward(self, x, batch, residual):
+    prepares_norm = True
+
+    def forward(self, x, batch, residual, then_norm=None):
         h = L.gated_linear(x, self.w13)
-        L.linear_into(h, self.w2, residual)
+        return L.linear_into(h, self.w2, residual, then_norm)
 
 
 register_feed_forward("gated", GatedFeedForward)

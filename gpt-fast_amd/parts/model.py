@@ -73,12 +73,24 @@ class DecoderModel:
     def forward(self, batch, cache) -> torch.Tensor:
         """float32 logits [n_wanted, vocab] of the step described by ``batch``."""
         residual = K.embed(self.embedding, batch.tokens)                  # model.py:140
-        for n, run in enumerate(self.plan.order):                         # model.py:142-143
-            self.blocks[run.layer].forward(residual, batch, cache.entries[n])
+        order = self.plan.order
+        x = None                       # rows of the next norm, if a block produced them
+        for n, run in enumerate(order):                                   # model.py:142-143
+            block = self.blocks[run.layer]
+            if not getattr(block, "prepares_norm", False):
+                block.forward(residual, batch, cache.entries[n])
+                x = None
+                continue
+            if n + 1 < len(order):
+                then_norm = getattr(self.blocks[order[n + 1].layer], "mixer_norm", None)
+            else:
+                then_norm = self.final_norm if getattr(batch, "every_row_wanted", False) else None
+            x = block.forward(residual, batch, cache.entries[n], x=x, then_norm=then_norm)
         if batch.n_want == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32,
                                device=residual.device)
-        x = self.final_norm.forward(residual, rows=batch.want_rows)       # model.py:144
+        if x is None:
+            x = self.final_norm.forward(residual, rows=batch.want_rows)   # model.py:144
         return L.linear(x, self.head, out_dtype=torch.float32)            # model.py:145
 
 

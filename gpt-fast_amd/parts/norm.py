@@ -26,5 +26,11 @@ class RMSNorm(Part):
     def forward(self, residual: torch.Tensor, rows=None) -> torch.Tensor:
         return K.rmsnorm(residual, self.weight, self.spec.eps, self.rt.dtype, rows=rows)
 
+    def row_and_column_form(self):
+        """This norm is a factor per row, rsqrt(mean(x^2) + eps), times a weight per column:
+        (column weights, eps).  A kernel that completes the residual stream can apply it in
+        the same pass."""
+        return self.weight, self.spec.eps
+
 
 register_norm("rms", RMSNorm)

@@ -51,6 +51,26 @@ def test_rmsnorm(dim, eps):
     close(out, tiny / math.sqrt(1e-8 + 1e-2), 1e-5)
 
 
+@pytest.mark.parametrize("rows,dim,eps", [(3, 72, 1e-5), (40, 200, 1e-6), (17, 4096, 1e-5),
+                                          (5, 6144, 1e-5), (9, 1001, 0.3)])
+def test_residual_sum_and_rmsnorm_in_one_pass(rows, dim, eps):
+    torch.manual_seed(12)
+    res0 = torch.randn(rows, dim, device=DEV) * 3
+    res0[0] *= 40.0
+    y = bf(torch.randn(rows, dim, device=DEV))
+    g = 1 + 0.1 * torch.randn(dim, device=DEV)
+    res = res0.clone()
+    out = K().add_rmsnorm(res, y, g, eps)
+    want_res = res0 + y.float()
+    assert torch.equal(res, want_res)
+    r = want_res.double()
+    close(out, r * torch.rsqrt((r ** 2).mean(-1, keepdim=True) + eps) * g.double(), 6e-3)
+    # the two separate kernels give the same rows
+    sep = res0.clone()
+    K().add_into(sep, y)
+    close(out, K().rmsnorm(sep, g, eps, torch.bfloat16), 6e-3)
+
+
 @pytest.mark.parametrize("M,N,K_", [(1, 5, 3), (3, 100, 70), (65, 130, 257), (200, 64, 1000)])
 def test_gemm_f32(M, N, K_):
     torch.manual_seed(2)

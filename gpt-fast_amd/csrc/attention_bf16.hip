@@ -289,12 +289,19 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
 #define TL_RT 2
 #define TL_ROWS (TL_WAVES * TL_RT * 16)
 
-template <int DS>
+// FULL: the head size is exactly the one the tiles are laid out for (no edge tests).
+// The running maximum of a row is only raised when a block's maximum exceeds it by more than
+// TL_SLACK (in log2 units): probabilities then stay below 2^TL_SLACK, which float sums and the
+// bfloat16 operand of the second product hold at full relative precision, and the output
+// accumulators are rescaled rarely instead of nearly every block.
+#define TL_SLACK 8.0f
+template <int DS, bool FULL>
 __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
-        bf16_t* __restrict__ out, int H, int Hkv, int hd, float scale_log2, int window) {
+        bf16_t* __restrict__ out, int H, int Hkv, int hd, float scale_log2, int window,
+        int pair_from) {
     constexpr int DT = DS * 2, RT = TL_RT;
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
     constexpr int KPITCH = HDM * 2 + 16;                  // bytes per key row in LDS
@@ -303,12 +310,25 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 x (K tile, V tile)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
-    const int g = blockIdx.y, seq = blockIdx.z;
+    const int seq = blockIdx.z;
     const int R = H / Hkv;
     const int q0 = q_start[seq];
     const int rows_total = (q_start[seq + 1] - q0) * R;
-    // later tiles see more keys: hand them out first so that the longest work starts first
-    const int wg_row0 = (gridDim.x - 1 - blockIdx.x) * TL_ROWS;
+    // Later tiles see more keys.  Workgroups are handed out in the order of their linear
+    // index; rank r in the order "most keys first" is tile gridDim.x - 1 - r / Hkv, head
+    // r % Hkv.  Ranks are given out in descending work; if all workgroups fit the chip at
+    // once (pair_from > 0: two per compute unit, index i + pair_from joining index i), the
+    // joining half takes the light ranks lightest first, so that every compute unit holds
+    // about the same number of keys.
+    const int total = gridDim.x * gridDim.y;
+    const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+    int rank = lin;
+    if (pair_from > 0) {
+        const int idx = (lin / (2 * pair_from)) * pair_from + lin % pair_from;
+        rank = ((lin / pair_from) & 1) ? total - 1 - idx : idx;
+    }
+    const int g = rank % gridDim.y;
+    const int wg_row0 = (gridDim.x - 1 - rank / gridDim.y) * TL_ROWS;
     if (wg_row0 >= rows_total) return;
     const int spos = start_pos[seq];
     const int* pages = table + (size_t)seq * table_stride;
@@ -328,7 +348,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const int d = ds * 32 + lg * 8;
-            qf[rt][ds].u = (valid && d < hd) ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
+            qf[rt][ds].u = (valid && (FULL || d < hd)) ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
         }
     }
     // key range of the workgroup and of this wave
@@ -356,47 +376,57 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     const int k_chunks = 64 * hd / 8, v_chunks = hd * 64 / 8;      // 16-byte pieces
     constexpr int K_PER = (64 * HDM / 8 + 255) / 256, V_PER = (HDM * 64 / 8 + 255) / 256;
     uint4 kreg[K_PER], vreg[V_PER];
+    int k_dst[K_PER], v_dst[V_PER];                        // LDS byte offsets of this thread's pieces
+    {
+        const int hd8 = hd / 8;                            // 16-byte pieces per key row
+#pragma unroll
+        for (int i = 0; i < K_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            const int key = c / hd8, piece = c - key * hd8;
+            k_dst[i] = (FULL || c < k_chunks) ? key * KPITCH + piece * 16 : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; ++i) {
+            const int c = threadIdx.x + i * 256;
+            v_dst[i] = (FULL || c < v_chunks) ? (c >> 3) * VPITCH + (c & 7) * 16 : -1;   // dim, 8 keys
+        }
+    }
     auto fetch_page = [&](int pg) {
         const int page = pages[pg];
         const uint4* ksrc = (const uint4*)(k_pages + page_row(page, g, 0, Hkv, hd));
         const uint4* vsrc = (const uint4*)(v_pages + value_elem(page, g, 0, 0, Hkv, hd));
 #pragma unroll
-        for (int i = 0; i < K_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            kreg[i] = c < k_chunks ? ksrc[c] : make_uint4(0, 0, 0, 0);
-        }
+        for (int i = 0; i < K_PER; ++i)
+            kreg[i] = k_dst[i] >= 0 ? ksrc[threadIdx.x + i * 256] : make_uint4(0, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i < V_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            vreg[i] = c < v_chunks ? vsrc[c] : make_uint4(0, 0, 0, 0);
-        }
+        for (int i = 0; i < V_PER; ++i)
+            vreg[i] = v_dst[i] >= 0 ? vsrc[threadIdx.x + i * 256] : make_uint4(0, 0, 0, 0);
     };
     auto store_page = [&](int buf, int pg) {
         char* kt = smem + buf * (KBYTES + VBYTES);
         char* vt = kt + KBYTES;
-        const int hd8 = hd / 8;                            // 16-byte pieces per key row
         const int keys_ok = wg_pmax - pg * 64;             // keys beyond hold no data yet
 #pragma unroll
-        for (int i = 0; i < K_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            if (c < k_chunks) {
-                const int key = c / hd8, piece = c - key * hd8;
-                *(uint4*)(kt + key * KPITCH + piece * 16) = kreg[i];
+        for (int i = 0; i < K_PER; ++i)
+            if (k_dst[i] >= 0) *(uint4*)(kt + k_dst[i]) = kreg[i];
+        if (keys_ok < 63) {                                // the last page: zero what is not data
+#pragma unroll
+            for (int i = 0; i < V_PER; ++i) {
+                const int piece = (threadIdx.x + i * 256) & 7;
+                Frag f;
+                f.u = vreg[i];
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (piece * 8 + e > keys_ok) f.e[e] = 0;
+                vreg[i] = f.u;
             }
         }
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            if (c < v_chunks) {
-                const int d = c >> 3, piece = c & 7;       // 8 pieces of 8 keys per dim
+            if (v_dst[i] >= 0) {
                 Frag f;
                 f.u = vreg[i];
-                if (piece * 8 + 7 > keys_ok) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (piece * 8 + e > keys_ok) f.e[e] = 0;
-                }
-                uint2* dst = (uint2*)(vt + d * VPITCH + piece * 16);
+                uint2* dst = (uint2*)(vt + v_dst[i]);
                 dst[0] = f.h[0];
                 dst[1] = f.h[1];
             }
@@ -413,7 +443,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
             Frag kf[DS];
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds)
-                kf[ds].u = (ds * 32 + lg * 8 < hd)
+                kf[ds].u = (FULL || ds * 32 + lg * 8 < hd)
                                ? *(const uint4*)(kt + (in_page + kt16 * 16 + li) * KPITCH + (ds * 32 + lg * 8) * 2)
                                : make_uint4(0, 0, 0, 0);
 #pragma unroll
@@ -426,56 +456,54 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         }
         const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
         Frag pf[RT];
-        float alpha[RT];
-        bool rescale = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            float sv[8];
-            float mx = -INFINITY;
+            float sv[8];                                   // raw scores; -inf where masked
             if (masked) {
                 const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int key = key0 + (e >> 2) * 16 + (e & 3);
-                    const float v = s[rt][e >> 2][e & 3] * scale_log2;
-                    sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
-                    mx = fmaxf(mx, sv[e]);
+                    sv[e] = (key <= rpos[rt] && key >= first) ? s[rt][e >> 2][e & 3] : -INFINITY;
                 }
             } else {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    sv[e] = s[rt][e >> 2][e & 3] * scale_log2;
-                    mx = fmaxf(mx, sv[e]);
-                }
+                for (int e = 0; e < 8; ++e) sv[e] = s[rt][e >> 2][e & 3];
             }
+            float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                             fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m[rt], mx);
-            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - m_safe);
+            mx *= scale_log2;                              // scale > 0: the order is kept
+            if (__builtin_amdgcn_ballot_w64(mx > m[rt] + TL_SLACK) != 0) {
+                // some row's maximum moved far: raise every row's reference and rescale
+                const float m_new = fmaxf(m[rt], mx);
+                const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[rt] - m_new);
+                l[rt] *= alpha;
+                m[rt] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= alpha;
+            }
+            const float neg_m = (m[rt] == -INFINITY) ? 0.f : -m[rt];
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = __builtin_amdgcn_exp2f(sv[e] - m_safe);
+                const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], scale_log2, neg_m));
                 sum += p;
                 pf[rt].e[e] = float_to_bf16(p);
             }
-            l[rt] = l[rt] * alpha[rt] + sum;
-            m[rt] = m_new;
-            rescale = rescale || (__builtin_amdgcn_ballot_w64(alpha[rt] != 1.f) != 0);
+            l[rt] += sum;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            if (dt * 16 < hd) {
+            if (FULL || dt * 16 < hd) {
                 Frag vf;
                 const char* vrow = vt + (dt * 16 + li) * VPITCH + (in_page + lg * 4) * 2;
                 vf.h[0] = *(const uint2*)vrow;
                 vf.h[1] = *(const uint2*)(vrow + 32);
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                    if (rescale) o[rt][dt] *= alpha[rt];
+                for (int rt = 0; rt < RT; ++rt)
                     o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][dt], 0, 0, 0);
-                }
             }
         }
     };
@@ -517,21 +545,30 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     }
 }
 
-template <int DS>
+template <int DS, bool FULL>
 static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k,
                                    const bf16_t* v, const int* q_start, const int* start_pos,
                                    const int* table, int table_stride, bf16_t* out, int H, int Hkv,
                                    int hd, float sl2, int window) {
     constexpr int HDM = DS * 32;
+    static int slots = 0;                                  // workgroups the chip holds at once
+    if (slots == 0) {
+        int dev = 0, cus = 0;
+        hipGetDevice(&dev);
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        slots = 2 * (cus > 0 ? cus : 1);
+    }
+    const int total = (int)(grid.x * grid.y);
+    const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
     const size_t shmem = 2 * (size_t)(64 * (HDM * 2 + 16) + HDM * (64 * 2 + 8));
     static bool raised = false;
     if (!raised) {
-        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS>,
+        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         raised = true;
     }
-    attention_tiled_kernel<DS><<<grid, 256, shmem, stream>>>(q, k, v, q_start, start_pos, table,
-                                                             table_stride, out, H, Hkv, hd, sl2, window);
+    attention_tiled_kernel<DS, FULL><<<grid, 256, shmem, stream>>>(q, k, v, q_start, start_pos, table,
+                                                             table_stride, out, H, Hkv, hd, sl2, window, pair_from);
 }
 
 // Prompts of many rows: max_tiles = most 128-row tiles any sequence needs per kv head.
@@ -544,10 +581,10 @@ extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, cons
     if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_tiles < 1) return (int)hipErrorInvalidValue;
     const dim3 grid(max_tiles, Hkv, n_seqs);
     const float sl2 = scale * LOG2E;
-    if (hd <= 64)
-        launch_attention_tiled<2>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
-    else
-        launch_attention_tiled<4>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    if (hd == 64) launch_attention_tiled<2, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    else if (hd < 64) launch_attention_tiled<2, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    else if (hd == 128) launch_attention_tiled<4, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    else launch_attention_tiled<4, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
     return GFA_LAUNCH_RESULT();
 }
 

@@ -7,7 +7,8 @@ product; one fused-multiply-add chain per output).
 bfloat16 engine: hand-written kernels for the few-row products of decoding (up to 16
 rows; weights are streamed once; see csrc/gemm_bf16.hip); the vendor matrix library,
 through ``torch.matmul``, for products of more rows - the reference uses the vendor
-library for these as well.  Accumulation is float32 everywhere.
+library for these as well - except where a hand-written kernel for 17..64 rows
+(csrc/gemm_wide_bf16.hip) measures faster.  Accumulation is float32 everywhere.
 """
 from typing import Optional
 
@@ -48,11 +49,26 @@ def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_n
     factor per row times a weight per column, sum and norm run as one pass and the normed
     rows are returned; else None, and the caller runs the norm."""
     form = getattr(then_norm, "row_and_column_form", None)
-    if form is not None and x.dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS:
-        weight, eps = form()
-        return K.add_rmsnorm(residual, torch.matmul(x, w.t()), weight, eps)
+    if x.dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS:
+        weight, eps = form() if form is not None else (None, 0.0)
+        if _sliced_is_faster(x.shape[0], w.shape[0], x.shape[1]):
+            return _wide().product_into(x, w, residual, weight, eps)
+        if form is not None:
+            return K.add_rmsnorm(residual, torch.matmul(x, w.t()), weight, eps)
     _linear_into(x, w, residual)
     return None
+
+
+def _wide():
+    from . import gemm_wide_bf16
+    return gemm_wide_bf16
+
+
+def _sliced_is_faster(M: int, N: int, K_: int) -> bool:
+    """17..64 rows times a matrix with few rows and a long inner size (the feed-forward's
+    second product): the hand-written kernel cuts K into slices over many workgroups where
+    the vendor library runs few; measured faster from an inner size of twice the width."""
+    return M <= _wide().MAX_ROWS and K_ % 8 == 0 and N % 4 == 0 and N <= 16384 and K_ >= 2 * N
 
 
 def _linear_into(x, w, residual):

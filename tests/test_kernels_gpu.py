@@ -108,6 +108,55 @@ def test_skinny_bf16(M, N, K_):
         close(G.skinny_gated(x, w), (g * torch.sigmoid(g)) * ref[:, I:], 1.5e-2)
 
 
+@pytest.mark.parametrize("M", [3, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K_", [(40, 64), (136, 200), (1000, 328), (256, 4096), (77, 72), (4096, 1024)])
+def test_products_of_up_to_64_rows(M, N, K_):
+    """The kernels for 17..64 rows (shared x in LDS, K in slices): plain, float, into the
+    residual stream with and without the norm that follows, and gated."""
+    from gpt_fast_amd.ops import gemm_wide_bf16 as W
+    torch.manual_seed(14)
+    x = bf(torch.randn(M, K_, device=DEV))
+    w = bf(torch.randn(N, K_, device=DEV) * 0.1)
+    ref = x.double() @ w.double().T
+    close(W.product(x, w, torch.float32), ref, 2e-5 if W.slices(M, N, K_) == 1 else 2e-5)
+    close(W.product(x, w), ref, 6e-3)
+    res0 = torch.randn(M, N, device=DEV)
+    res = res0.clone()
+    assert W.product_into(x, w, res) is None
+    close(res, res0.double() + ref, 2e-5)
+    if N % 4 == 0:
+        g = 1 + 0.1 * torch.randn(N, device=DEV)
+        res2 = res0.clone()
+        xn = W.product_into(x, w, res2, g, 1e-5)
+        close(res2, res0.double() + ref, 2e-5)
+        if xn is not None:                                 # sliced: the norm rode along
+            assert W.slices(M, N, K_) > 1
+            r = res2.double()
+            close(xn, r * torch.rsqrt((r ** 2).mean(-1, keepdim=True) + 1e-5) * g.double(), 6e-3)
+    if N % 2 == 0:
+        I = N // 2
+        a = ref[:, :I]
+        close(W.product_gated(x, w), (a * torch.sigmoid(a)) * ref[:, I:], 1e-2)
+
+
+def test_sliced_product_equals_its_slices_added_in_order():
+    from gpt_fast_amd.ops import gemm_wide_bf16 as W
+    torch.manual_seed(15)
+    M, N, K_ = 40, 512, 4096
+    x = bf(torch.randn(M, K_, device=DEV))
+    w = bf(torch.randn(N, K_, device=DEV) * 0.1)
+    part = W.partial_sums(x, w)
+    S = part.shape[0]
+    assert S == W.slices(M, N, K_) and S > 1
+    total = part[0].clone()
+    for s in range(1, S):
+        total += part[s]
+    assert torch.equal(W.sum_store(part, torch.float32), total)
+    per = ((K_ + 127) // 128 + S - 1) // S * 128
+    for s in (0, S - 1):
+        close(part[s], x[:, s * per:(s + 1) * per].double() @ w[:, s * per:(s + 1) * per].double().T, 2e-5)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_silu_mul_and_add_into(dtype):
     torch.manual_seed(4)

@@ -100,6 +100,7 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
+    ap.add_argument("--batch", type=int, default=8, help="sequences decoded together (headline: 8)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
     args = ap.parse_args()
@@ -116,7 +117,7 @@ def main():
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     cfg = LlamaConfig.from_dict(raw)
-    batch, context, prompt_len = 8, 4096, 128
+    batch, context, prompt_len = args.batch, 4096, 128
     t0 = time.time()
     engine = gfa.Engine.from_random("llama", cfg, seed=0, dtype="bfloat16", device="cuda:0",
                                     max_tokens=64 * context, max_sequences=64)
@@ -128,7 +129,7 @@ def main():
     value = batch / dt
     log(f"[bench] decode b{batch}: {dt * 1e3:.3f} ms/step, {value:.1f} tok/s")
     out = {
-        "metric": "decode tok/s @ batch 8; Llama-3.1-8B bf16", "value": round(value, 2),
+        "metric": f"decode tok/s @ batch {batch}; Llama-3.1-8B bf16", "value": round(value, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / BASELINE_TOK_S, 3), "dtype": "bf16", "data": "synthetic",

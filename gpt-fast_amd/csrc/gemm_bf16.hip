@@ -353,6 +353,35 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     };
     if (t_begin < t_end) load_piece(t_begin, regs_a);
     if (t_begin + 1 < t_end) load_piece(t_begin + 1, regs_b);
+    // What the epilogue of wave 0 reads is requested now, behind the first pieces of W, so
+    // that its latency (and the rotation's sine and cosine) passes while W streams.
+    float4 res_pre[CT];                                  // MODE 2: the residual's old values
+    bool res_ok[CT];
+    float rot_cs[2] = {1.f, 1.f}, rot_sn[2] = {0.f, 0.f};   // MODE 4, one tile of rows
+    int rot_pos = 0, rot_page = 0;
+    constexpr bool ROT_EARLY = MODE == 4 && CT == 1;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        res_ok[ct] = false;
+        if (MODE == 2 && wave == 0) {
+            const int m = ct * 16 + fi, n = n0 + fg * 4;
+            res_ok[ct] = m < M && n + 3 < N && (ldo & 3) == 0;
+            if (res_ok[ct]) res_pre[ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
+        }
+    }
+    if (ROT_EARLY && wave == 0 && fi < M && n0 + fg * 4 < N) {
+        const int n = n0 + fg * 4;
+        const int head = n / ex.hd, d = n - head * ex.hd;
+        rot_pos = ex.tok_pos[fi];
+        if (head >= ex.H && ex.k_pages)
+            rot_page = ex.table[(size_t)ex.tok_seq[fi] * ex.table_stride + rot_pos / GFA_PAGE];
+        if (head < ex.H + ex.Hkv) {
+#pragma unroll
+            for (int pr = 0; pr < 2; ++pr)
+                if (d + 2 * pr < ex.rot)
+                    sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[pr], &rot_cs[pr]);
+        }
+    }
     for (int t = t_begin; t < t_end; t += 2) {
         load_x(t);
         stage_piece(regs_a);
@@ -411,15 +440,15 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             const int n = n0 + fg * 4;
             if (n >= N) continue;
             const int hd = ex.hd, head = n / hd, d = n - head * hd;
-            const int pos = ex.tok_pos[m];
+            const int pos = ROT_EARLY ? rot_pos : ex.tok_pos[m];
             float v[4] = {acc[0][ct][0], acc[0][ct][1], acc[0][ct][2], acc[0][ct][3]};
             if (head < ex.H + ex.Hkv) {
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     const int dd = d + 2 * pr;
                     if (dd < ex.rot) {
-                        float sn, cs;
-                        sincosf((float)pos * ex.freqs[dd >> 1], &sn, &cs);
+                        float sn = rot_sn[pr], cs = rot_cs[pr];
+                        if (!ROT_EARLY) sincosf((float)pos * ex.freqs[dd >> 1], &sn, &cs);
                         const float a = v[2 * pr], bb = v[2 * pr + 1];
                         v[2 * pr] = a * cs - bb * sn;
                         v[2 * pr + 1] = bb * cs + a * sn;
@@ -433,7 +462,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             if (head < ex.H) {
                 *(uint2*)(ex.q_out + ((size_t)m * ex.H + head) * hd + d) = make_uint2(pk.u.x, pk.u.y);
             } else if (ex.k_pages) {
-                const int page = ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + pos / GFA_PAGE];
+                const int page = ROT_EARLY ? rot_page
+                    : ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + pos / GFA_PAGE];
                 const int off = pos % GFA_PAGE;
                 if (head < ex.H + ex.Hkv) {
                     *(uint2*)(ex.k_pages + page_row(page, head - ex.H, off, ex.Hkv, hd) + d) =
@@ -445,6 +475,13 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                         ex.v_pages[value_elem(page, g, d + j, off, ex.Hkv, hd)] = e[j];
                 }
             }
+        } else if (MODE == 2 && res_ok[ct]) {
+            float4 r = res_pre[ct];                      // the same sums as skinny_store<2>
+            r.x += acc[0][ct][0];
+            r.y += acc[0][ct][1];
+            r.z += acc[0][ct][2];
+            r.w += acc[0][ct][3];
+            *(float4*)((float*)out + (size_t)m * ldo + n0 + fg * 4) = r;
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {

@@ -48,7 +48,7 @@ def replay(engine: Engine, lines, out_dir: str, log=None) -> int:
                 data = logits.detach().to("cpu", torch.float32).contiguous().numpy()
                 path = os.path.join(out_dir, f"{step}.f32")
                 with open(path + ".tmp", "wb") as f:
-                    f.write(data.astype("<f4", copy=False).tobytes())
+                    data.astype("<f4", copy=False).tofile(f)
                 os.replace(path + ".tmp", path)
             else:
                 torch.cuda.synchronize()

@@ -36,7 +36,7 @@ class Engine:
         self.rt = model.rt
         pages = (max_tokens + PAGE - 1) // PAGE
         if max_sequences is None:
-            max_sequences = min(pages, 1024)
+            max_sequences = pages                 # a live sequence holds at least one page
         self.cache = Cache(model.cache_needs(), model.cache_borrow(), max_tokens=max_tokens,
                            max_sequences=max_sequences, dtype=self.rt.dtype, device=self.rt.device)
         self.uploader = BatchUploader(self.rt.device)

@@ -240,6 +240,18 @@ struct SkinnyExtra {
     const int* tok_pos;
     const int* table;
     int table_stride, H, Hkv, hd, rot;
+    // A norm spread over two kernels (one tile of rows).  The kernel that completes the
+    // residual stream (MODE 2) also writes xg_out [M, N] = bfloat16(new residual * next_g) and
+    // ssq_out [tiles, 16]: each workgroup's share of its 16 rows' sums of squares (float, from
+    // the float residual).  The next product takes xg as its x, adds the shares in a fixed
+    // order (ssq_in [t_in, 16]) and scales its result by rsqrt(sum / K + eps): a factor per row
+    // commutes with the product, so this is the RMS norm of model.py:236-241.
+    bf16_t* xg_out;
+    const float* next_g;
+    float* ssq_out;
+    const float* ssq_in;
+    int t_in;
+    int share_off;            // byte offset in LDS of the waves' pieces for the shares
 };
 
 template <int CT, int MODE, bool NORM>
@@ -355,7 +367,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     if (t_begin + 1 < t_end) load_piece(t_begin + 1, regs_b);
     // What the epilogue of wave 0 reads is requested now, behind the first pieces of W, so
     // that its latency (and the rotation's sine and cosine) passes while W streams.
-    float4 res_pre[CT];                                  // MODE 2: the residual's old values
+    float4 res_pre[CT], g_pre[CT];                       // MODE 2: the residual's old values, next norm's weights
     bool res_ok[CT];
     float rot_cs[2] = {1.f, 1.f}, rot_sn[2] = {0.f, 0.f};   // MODE 4, one tile of rows
     int rot_pos = 0, rot_page = 0;
@@ -366,7 +378,10 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         if (MODE == 2 && wave == 0) {
             const int m = ct * 16 + fi, n = n0 + fg * 4;
             res_ok[ct] = m < M && n + 3 < N && (ldo & 3) == 0;
-            if (res_ok[ct]) res_pre[ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
+            if (res_ok[ct]) {
+                res_pre[ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
+                if (ex.xg_out) g_pre[ct] = *(const float4*)(ex.next_g + n);
+            }
         }
     }
     if (ROT_EARLY && wave == 0 && fi < M && n0 + fg * 4 < N) {
@@ -380,6 +395,25 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int pr = 0; pr < 2; ++pr)
                 if (d + 2 * pr < ex.rot)
                     sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[pr], &rot_cs[pr]);
+        }
+    }
+    // second half of a two-kernel norm: lane group fg of wave w takes the shares of the
+    // column tiles fg + 4 w, + 4 NW ..., 16 rows side by side (64 contiguous bytes each).
+    // They are requested here as copies straight into a wave-private piece of LDS - no
+    // register waits for them, so nothing below is held up - and added after the product.
+    constexpr int SHARES = 16;
+    const bool chained = CT == 1 && ex.ssq_in != nullptr;
+    float* share_lds = (float*)(smem + ex.share_off) + wave * (SHARES * 64);
+    if (chained) {
+#pragma unroll
+        for (int j = 0; j < SHARES; ++j) {
+            const int tile = fg + 4 * (wave + NW * j);
+            if (4 * (wave + NW * j) < ex.t_in) {          // wave-uniform
+                const float* src = ex.ssq_in + (size_t)(tile < ex.t_in ? tile : 0) * 16 + fi;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)src,
+                    (__attribute__((address_space(3))) void*)(share_lds + j * 64), 4, 0, 0);
+            }
         }
     }
     for (int t = t_begin; t < t_end; t += 2) {
@@ -401,6 +435,22 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             ssq[ct] += __shfl_xor(ssq[ct], 32, GFA_WAVE);
         }
     }
+    if (chained) {                                       // fixed order: lane, lane groups, waves
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the copies into LDS have landed
+        float pre_ssq = 0.f;
+#pragma unroll
+        for (int j = 0; j < SHARES; ++j) {
+            const int tile = fg + 4 * (wave + NW * j);
+            if (tile < ex.t_in) pre_ssq += share_lds[j * 64 + lane];
+        }
+        for (int tile = fg + 4 * (wave + NW * SHARES); tile < ex.t_in; tile += 4 * NW)
+            pre_ssq += ex.ssq_in[(size_t)tile * 16 + fi];
+        const float other = __shfl_xor(pre_ssq, 16, GFA_WAVE);
+        pre_ssq = (fg & 1) ? other + pre_ssq : pre_ssq + other;      // (g0 + g1), (g2 + g3)
+        const float pair = __shfl_xor(pre_ssq, 32, GFA_WAVE);
+        pre_ssq = (fg & 2) ? pair + pre_ssq : pre_ssq + pair;        // (g0 + g1) + (g2 + g3)
+        ssq[0] = pre_ssq;                                // from here on as the fused norm's sum
+    }
     if (NW > 1) {
         __syncthreads();                                 // staging is done; reuse it for the sums
         floatx4_t* red = (floatx4_t*)smem;
@@ -409,7 +459,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) red[((wave * RT + rt) * CT + ct) * 64 + lane] = acc[rt][ct];
-        if (NORM && fg == 0) {
+        if ((NORM || chained) && fg == 0) {
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) red_s[(wave * CT + ct) * 16 + fi] = ssq[ct];
         }
@@ -420,17 +470,18 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += red[((wv * RT + rt) * CT + ct) * 64 + lane];
-            if (NORM) {
+            if (NORM || chained) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) ssq[ct] += red_s[(wv * CT + ct) * 16 + fi];
             }
         }
     }
+    float part_ssq = 0.f;                                // MODE 2 with xg_out: this lane's r^2
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = ct * 16 + fi;
         if (m >= M) continue;
-        if (NORM) {
+        if (NORM || chained) {
             const float rs = rsqrtf(ssq[ct] / (float)K + ex.eps);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) acc[rt][ct] *= rs;
@@ -482,6 +533,17 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             r.z += acc[0][ct][2];
             r.w += acc[0][ct][3];
             *(float4*)((float*)out + (size_t)m * ldo + n0 + fg * 4) = r;
+            if (ex.xg_out) {                             // first half of the next norm; N == ldo
+                const float4 g = g_pre[ct];
+                Frag8 pk;
+                bf16_t* e = (bf16_t*)&pk.u;
+                e[0] = float_to_bf16(r.x * g.x);
+                e[1] = float_to_bf16(r.y * g.y);
+                e[2] = float_to_bf16(r.z * g.z);
+                e[3] = float_to_bf16(r.w * g.w);
+                *(uint2*)(ex.xg_out + (size_t)m * ldo + n0 + fg * 4) = make_uint2(pk.u.x, pk.u.y);
+                part_ssq = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -489,6 +551,11 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                 if (n < N) skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
             }
         }
+    }
+    if (MODE == 2 && ex.xg_out) {                        // this workgroup's share, rows side by side
+        part_ssq += __shfl_xor(part_ssq, 16, GFA_WAVE);
+        part_ssq += __shfl_xor(part_ssq, 32, GFA_WAVE);
+        if (fg == 0) ex.ssq_out[(size_t)blockIdx.x * 16 + fi] = part_ssq;
     }
 }
 
@@ -511,6 +578,11 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         const size_t r2 = (size_t)nw * RT * ct * 64 * sizeof(floatx4_t) + (size_t)nw * ct * 16 * sizeof(float);
         if (nw > 1 && r2 > shmem) shmem = r2;
     }
+    SkinnyExtra exl = ex;
+    if (ex.ssq_in) {                                     // the waves' pieces for the norm's shares
+        exl.share_off = (int)shmem;
+        shmem += (size_t)nw * 16 * 64 * sizeof(float);
+    }
 #define GFA_LAUNCH_MFMA(CTV)                                                                      \
     do {                                                                                          \
         static bool raised = false;                                                               \
@@ -519,7 +591,7 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, NORM><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, ex); \
+        skinny_mfma_kernel<CTV, MODE, NORM><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
     } while (0)
     if (NORM) {                                          // the fused norm serves one 16-row tile
         if (ct != 1) return (int)hipErrorInvalidValue;
@@ -574,9 +646,11 @@ extern "C" int gfa_skinny_norm_bf16(const float* x_f32, const float* norm_w, flo
 
 // norm -> fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
 // w [(H + 2 Hkv) hd, K]; head size a multiple of 16, rotary width even, interleaved pairs.
-// Either x_f32 with its norm (x_bf16 null), or x_bf16 already normed (up to 64 rows).
+// Either x_f32 with its norm (x_bf16 null), or x_bf16 already normed (up to 64 rows), or
+// x_bf16 with ssq_in [t_in, 16]: the two halves of a norm that gfa_skinny_into_chain_bf16
+// left (eps the norm's; up to 16 rows).
 extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, float eps,
-                                       const void* x_bf16,
+                                       const void* x_bf16, const float* ssq_in, int t_in,
                                        const void* w, void* q_out, void* k_pages, void* v_pages,
                                        const float* freqs, const int* tok_seq, const int* tok_pos,
                                        const int* table, int table_stride, int M, int K, int H,
@@ -600,10 +674,52 @@ extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, 
     ex.Hkv = Hkv;
     ex.hd = hd;
     ex.rot = rot;
+    if (x_bf16 && ssq_in) {                               // second half of a two-kernel norm
+        if (M > 16 || t_in <= 0) return (int)hipErrorInvalidValue;
+        ex.ssq_in = ssq_in;
+        ex.t_in = t_in;
+    }
     const int N = (H + 2 * Hkv) * hd;
     if (x_bf16)
         return launch_skinny_mfma<4, false>((const bf16_t*)x_bf16, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
     return launch_skinny_mfma<4, true>(nullptr, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
+}
+
+// residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
+// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [(N + 15) / 16, 16] = the
+// workgroups' shares of the rows' sums of squares.  N a multiple of 4.
+extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* residual, int M,
+                                          int N, int K, const float* next_g, void* xg_out,
+                                          float* ssq_out, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0 || N % 4 != 0 || !next_g || !xg_out || !ssq_out)
+        return (int)hipErrorInvalidValue;
+    SkinnyExtra ex = {};
+    ex.next_g = next_g;
+    ex.xg_out = (bf16_t*)xg_out;
+    ex.ssq_out = ssq_out;
+    return launch_skinny_mfma<2, false>((const bf16_t*)x, (const bf16_t*)w, residual, M, N, K, N, 0, ex, stream);
+}
+
+// The product that follows: x = xg [M <= 16, K], the result scaled by
+// rsqrt(sum of ssq_in[:, m] / K + eps).  mode 0 bfloat16 out, 1 float out, 3 gate.
+extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, int t_in, float eps,
+                                           const void* w, void* out, int M, int N, int K, int ldo,
+                                           int mode, int gate_rows, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0 || !ssq_in || t_in <= 0) return (int)hipErrorInvalidValue;
+    SkinnyExtra ex = {};
+    ex.ssq_in = ssq_in;
+    ex.t_in = t_in;
+    ex.eps = eps;
+    const bf16_t* xp = (const bf16_t*)xg;
+    const bf16_t* wp = (const bf16_t*)w;
+    switch (mode) {
+        case 0: return launch_skinny_mfma<0, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 1: return launch_skinny_mfma<1, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 3: return launch_skinny_mfma<3, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+    }
+    return (int)hipErrorInvalidValue;
 }
 
 // x [M, K], w [N, K] (gate mode: [2 * N, K], gate_rows = N), out [M, ldo].

@@ -74,6 +74,72 @@ def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor]
     return out
 
 
+def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:
+    """The residual-completing product of this shape can prepare the norm that follows."""
+    return 0 < n_rows <= 16 and n_out % 8 == 0 and inner % 8 == 0
+
+
+def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
+                      next_g: torch.Tensor):
+    """residual += x w^T, and the first half of the RMS norm that follows: returns
+    ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, 16]: per
+    workgroup (16 columns) its share of each row's sum of squares.  Up to 16 rows."""
+    _check_operands(x, w, "skinny_into_chain")
+    M, K = x.shape
+    N = w.shape[0]
+    require_device(residual, next_g)
+    if residual.shape != (M, N) or residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("skinny_into_chain: residual must be contiguous float32 [M, N]")
+    if next_g.dtype != torch.float32 or next_g.numel() != N or not next_g.is_contiguous():
+        raise KernelError("skinny_into_chain: one float32 norm weight per column")
+    if not can_chain_norm(M, N, K):
+        raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
+    xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    ssq = torch.empty(((N + 15) // 16, 16), dtype=torch.float32, device=x.device)
+    check(library("gemm_bf16").gfa_skinny_into_chain_bf16(
+        ptr(x), ptr(w), ptr(residual), _i(M), _i(N), _i(K), ptr(next_g), ptr(xg), ptr(ssq),
+        stream_handle()), "skinny_into_chain")
+    return xg, ssq
+
+
+def _check_chain(xg, ssq, w, what):
+    _check_operands(xg, w, what)
+    require_device(ssq)
+    if xg.shape[0] > 16 or w.shape[1] % 8:
+        raise KernelError(f"{what}: takes 1..16 rows and an inner size that is a multiple of 8")
+    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[1] != 16 or not ssq.is_contiguous():
+        raise KernelError(f"{what}: ssq must be contiguous float32 [shares, 16]")
+
+
+def skinny_after_chain(xg, ssq, eps: float, w, out_dtype=torch.bfloat16):
+    """The second half: (xg w^T) scaled per row m by rsqrt(sum(ssq[:, m]) / K + eps)."""
+    _check_chain(xg, ssq, w, "skinny_after_chain")
+    M, K = xg.shape
+    N = w.shape[0]
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"skinny_after_chain: output type {out_dtype}")
+    out = torch.empty((M, N), dtype=out_dtype, device=w.device)
+    check(library("gemm_bf16").gfa_skinny_after_chain_bf16(
+        ptr(xg), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w), ptr(out), _i(M), _i(N),
+        _i(K), _i(N), _i(0 if out_dtype == torch.bfloat16 else 1), _i(0), stream_handle()),
+        "skinny_after_chain")
+    return out
+
+
+def skinny_after_chain_gated(xg, ssq, eps: float, w13):
+    """silu(n W1^T) * (n W3^T) with n the normed rows given by their two halves."""
+    _check_chain(xg, ssq, w13, "skinny_after_chain_gated")
+    M, K = xg.shape
+    if w13.shape[0] % 2:
+        raise KernelError("skinny_after_chain_gated: w13 needs an even number of rows")
+    I = w13.shape[0] // 2
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
+    check(library("gemm_bf16").gfa_skinny_after_chain_bf16(
+        ptr(xg), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I),
+        _i(K), _i(I), _i(3), _i(I), stream_handle()), "skinny_after_chain_gated")
+    return out
+
+
 def wide_f32_out(x: torch.Tensor, w: torch.Tensor):
     """Many rows, float32 result (logits of every position of a prompt): the vendor
     library with a float32 output; products of bfloat16 values are exact in float32 and
@@ -137,14 +203,19 @@ def skinny_normed_gated(x_f32, norm_w, eps: float, w13):
 
 
 def qkv_rope_store(x, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, k_pages,
-                   v_pages, n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int):
+                   v_pages, n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int,
+                   ssq: Optional[torch.Tensor] = None):
     """Fused q/k/v projection, rotation of interleaved pairs and the cache write in one
     kernel; returns q [M, H, hd].  ``x`` is either the float32 residual stream, read
     through the RMS norm (``norm_w``, ``eps``; up to 16 rows), or bfloat16 rows that are
-    normed already (``norm_w`` None; up to 64 rows).  k_pages None: nothing is stored."""
+    normed already (``norm_w`` None; up to 64 rows), or with ``ssq`` the two halves of a
+    norm as :func:`skinny_into_chain` leaves them (``eps`` the norm's; up to 16 rows).
+    k_pages None: nothing is stored."""
     fused_norm = x.dtype == torch.float32
     if fused_norm:
         _check_normed(x, norm_w, wqkv, "qkv_rope_store")
+    elif ssq is not None:
+        _check_chain(x, ssq, wqkv, "qkv_rope_store")
     else:
         _check_operands(x, wqkv, "qkv_rope_store")
         if wqkv.shape[1] % 8:
@@ -174,7 +245,8 @@ def qkv_rope_store(x, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, 
     q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=wqkv.device)
     check(library("gemm_bf16").gfa_qkv_rope_store_bf16(
         ptr(x if fused_norm else None), ptr(norm_w if fused_norm else None),
-        ctypes.c_float(eps if fused_norm else 0.0), ptr(None if fused_norm else x), ptr(wqkv),
+        ctypes.c_float(eps if fused_norm or ssq is not None else 0.0),
+        ptr(None if fused_norm else x), ptr(ssq), _i(0 if ssq is None else ssq.shape[0]), ptr(wqkv),
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table),
         _i(table.shape[1]), _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim),
         _i(rotary_dim), stream_handle()), "qkv_rope_store")

@@ -28,9 +28,40 @@ def _fast():
     return gemm_bf16
 
 
+class HalfNormed:
+    """Rows of an RMS norm in two halves, as the few-row product that completed the residual
+    stream left them: ``xg`` = bfloat16(residual * norm weight) [M, D] and ``ssq`` [shares, 16],
+    whose column sums are the rows' sums of squares (float32, from the float32 residual).
+    The products of this module take it in place of x and apply the missing factor
+    rsqrt(sum / D + eps) to their float32 result; a factor per row commutes with the product,
+    so this is the norm of model.py:236-241 with the rounding to bfloat16 before the row
+    factor instead of after it.  No kernel runs between the two products."""
+
+    __slots__ = ("xg", "ssq", "eps")
+
+    def __init__(self, xg, ssq, eps):
+        self.xg, self.ssq, self.eps = xg, ssq, eps
+
+    @property
+    def shape(self):
+        return self.xg.shape
+
+    @property
+    def dtype(self):
+        return self.xg.dtype
+
+    def materialize(self) -> torch.Tensor:
+        """The normed rows as an ordinary tensor (for a consumer that is no product here)."""
+        M, D = self.xg.shape
+        rs = torch.rsqrt(self.ssq.sum(dim=0)[:M, None] / D + self.eps)
+        return (self.xg.float() * rs).to(self.xg.dtype)
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
     """[M, N] = x [M, K] times w [N, K] transposed, in ``out_dtype`` (default: x's)."""
     out_dtype = out_dtype or x.dtype
+    if isinstance(x, HalfNormed):
+        return _fast().skinny_after_chain(x.xg, x.ssq, x.eps, w, out_dtype=out_dtype)
     if x.dtype == torch.float32:
         if out_dtype != torch.float32:
             raise KernelError("a float32 product has a float32 result")
@@ -43,12 +74,20 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return torch.matmul(x, w.t())
 
 
-def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_norm=None):
+def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_norm=None,
+                takes_halves: bool = False):
     """residual (float32 [M, N]) += x W^T.  ``then_norm``: the norm that reads the residual
     stream next.  Where the sum is a kernel of its own (many bfloat16 rows) and the norm is a
     factor per row times a weight per column, sum and norm run as one pass and the normed
-    rows are returned; else None, and the caller runs the norm."""
+    rows are returned; with few rows and ``takes_halves`` (the reader of the norm is a product
+    of this module) they are returned as a :class:`HalfNormed`; else None, and the caller runs
+    the norm."""
     form = getattr(then_norm, "row_and_column_form", None)
+    if (form is not None and takes_halves and x.dtype == torch.bfloat16
+            and _fast().can_chain_norm(x.shape[0], w.shape[0], x.shape[1])):
+        weight, eps = form()
+        xg, ssq = _fast().skinny_into_chain(x, w, residual, weight)
+        return HalfNormed(xg, ssq, eps)
     if x.dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS:
         weight, eps = form() if form is not None else (None, 0.0)
         if _sliced_is_faster(x.shape[0], w.shape[0], x.shape[1]):
@@ -82,6 +121,8 @@ def _linear_into(x, w, residual):
 def gated_linear(x: torch.Tensor, w13: torch.Tensor):
     """[M, I] = silu(x W1^T) * (x W3^T), with w13 = rows of W1 then rows of W3
     (model.py:227)."""
+    if isinstance(x, HalfNormed):
+        return _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13)
     if x.dtype == torch.float32:
         return K.silu_mul(K.gemm_f32(x, w13))
     if x.shape[0] <= SKINNY_MAX_ROWS:
@@ -92,11 +133,18 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
 # ----------------------------------------------------------------------------- fused projection
 def can_project_rotate_store(x: torch.Tensor, wqkv: torch.Tensor, head_dim: int) -> bool:
     """True if the fused projection / rotation / cache-write kernel takes these rows."""
+    if isinstance(x, HalfNormed):
+        return head_dim % 16 == 0
     return (x.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
             and wqkv.shape[1] % 8 == 0 and head_dim % 16 == 0)
 
 
 def qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
                    n_heads, n_kv_heads, head_dim, rotary_dim):
+    if isinstance(residual, HalfNormed):
+        h = residual
+        return _fast().qkv_rope_store(h.xg, None, h.eps, wqkv, freqs, tok_seq, tok_pos, table,
+                                      k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotary_dim,
+                                      ssq=h.ssq)
     return _fast().qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table,
                                   k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotary_dim)

@@ -40,8 +40,9 @@ class Attention(Part):
         return KVNeed(s.n_kv_heads, s.head_dim, s.window)
 
     prepares_norm = True
+    takes_prepared = True          # x may be an ops.linear.HalfNormed
 
-    def forward(self, x, batch, entry, residual, then_norm=None):
+    def forward(self, x, batch, entry, residual, then_norm=None, takes_halves=False):
         s = self.spec
         q = None
         fused = getattr(self.position, "project_rotate_store", None)
@@ -55,7 +56,7 @@ class Attention(Part):
         y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
                         self.scale, self.window)                            # model.py:209-211
         return L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual,
-                             then_norm)                                     # model.py:215, 162
+                             then_norm, takes_halves)                       # model.py:215, 162
 
 
 register_mixer("attention", Attention)

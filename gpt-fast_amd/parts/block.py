@@ -38,23 +38,31 @@ class PreNormBlock(Part):
 
     # Norm hand-over, optional for every part: a mixer or feed-forward that sets
     # ``prepares_norm`` takes ``then_norm=`` (the norm that reads the residual stream after
-    # it) and returns that norm's rows if it produced them on the way, else None.  A block
-    # that sets it takes ``x=`` (the rows of its first norm, if the caller has them) and
-    # ``then_norm=`` in the same sense, and names its first norm ``mixer_norm``.
+    # it) and ``takes_halves=`` (whether that norm's reader accepts an ops.linear.HalfNormed
+    # in place of x; a part says so with ``takes_prepared``), and returns that norm's rows if
+    # it produced them on the way, else None.  A block that sets ``prepares_norm`` takes
+    # ``x=`` (the rows of its first norm, if the caller has them), ``then_norm=`` and
+    # ``takes_halves=`` in the same sense, and names its first norm ``mixer_norm``.
     prepares_norm = True
 
-    def forward(self, residual, batch, entry, x=None, then_norm=None):
+    @property
+    def takes_prepared(self):
+        return getattr(self.mixer, "takes_prepared", False)
+
+    def forward(self, residual, batch, entry, x=None, then_norm=None, takes_halves=False):
         if x is None:
             x = self.mixer_norm.forward(residual)
         h = None
         if getattr(self.mixer, "prepares_norm", False):
-            h = self.mixer.forward(x, batch, entry, residual, then_norm=self.feed_forward_norm)
+            h = self.mixer.forward(x, batch, entry, residual, then_norm=self.feed_forward_norm,
+                                   takes_halves=getattr(self.feed_forward, "takes_prepared", False))
         else:
             self.mixer.forward(x, batch, entry, residual)
         if h is None:
             h = self.feed_forward_norm.forward(residual)
         if then_norm is not None and getattr(self.feed_forward, "prepares_norm", False):
-            return self.feed_forward.forward(h, batch, residual, then_norm=then_norm)
+            return self.feed_forward.forward(h, batch, residual, then_norm=then_norm,
+                                             takes_halves=takes_halves)
         self.feed_forward.forward(h, batch, residual)
         return None
 

@@ -24,10 +24,11 @@ class GatedFeedForward(Part):
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
     prepares_norm = True
+    takes_prepared = True          # x may be an ops.linear.HalfNormed
 
-    def forward(self, x, batch, residual, then_norm=None):
+    def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
         h = L.gated_linear(x, self.w13)
-        return L.linear_into(h, self.w2, residual, then_norm)
+        return L.linear_into(h, self.w2, residual, then_norm, takes_halves)
 
 
 register_feed_forward("gated", GatedFeedForward)

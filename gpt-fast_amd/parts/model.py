@@ -81,11 +81,16 @@ class DecoderModel:
                 block.forward(residual, batch, cache.entries[n])
                 x = None
                 continue
+            takes_halves = True                    # the head is a product of ops.linear
             if n + 1 < len(order):
-                then_norm = getattr(self.blocks[order[n + 1].layer], "mixer_norm", None)
+                nxt = self.blocks[order[n + 1].layer]
+                then_norm = getattr(nxt, "mixer_norm", None)
+                takes_halves = (getattr(nxt, "prepares_norm", False)
+                                and getattr(nxt, "takes_prepared", False))
             else:
                 then_norm = self.final_norm if getattr(batch, "every_row_wanted", False) else None
-            x = block.forward(residual, batch, cache.entries[n], x=x, then_norm=then_norm)
+            x = block.forward(residual, batch, cache.entries[n], x=x, then_norm=then_norm,
+                              takes_halves=takes_halves)
         if batch.n_want == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32,
                                device=residual.device)

@@ -396,6 +396,45 @@ def test_products_fused_with_the_norm(M, N, K_, eps):
     close(G.skinny_normed(x, g, eps, w, out_dtype=torch.float32), unfused, 1e-2)
 
 
+@pytest.mark.parametrize("M", [1, 2, 5, 16])
+@pytest.mark.parametrize("D,K_,N2,eps", [(72, 40, 48, 1e-5), (200, 328, 208, 1e-6),
+                                         (4096, 1024, 256, 1e-5), (1000, 64, 96, 0.3),
+                                         (8192, 64, 64, 1e-5)])
+def test_norm_over_two_kernels(M, D, K_, N2, eps):
+    """The product that completes the residual stream prepares the next norm (column
+    weights applied, shares of the sums of squares); the next product applies the row
+    factor.  Against float64, and against the engine's own separate kernels."""
+    from gpt_fast_amd.ops import gemm_bf16 as G
+    torch.manual_seed(10)
+    res0 = torch.randn(M, D, device=DEV) * 3
+    res0[0] *= 50.0                                   # rows of very different size
+    y = bf(torch.randn(M, K_, device=DEV))
+    wo = bf(torch.randn(D, K_, device=DEV) * 0.2)
+    g = 1 + 0.1 * torch.randn(D, device=DEV)
+    w = bf(torch.randn(N2, D, device=DEV) * 0.1)
+    res = res0.clone()
+    xg, ssq = G.skinny_into_chain(y, wo, res, g)
+    res_ref = res0.double() + y.double() @ wo.double().T
+    close(res, res_ref, 1e-5)
+    close(ssq.sum(0)[:M], (res.double() ** 2).sum(1), 1e-5)
+    assert float(ssq[:, M:].abs().max()) == 0 if M < 16 else True
+    n = res.double() * torch.rsqrt((res.double() ** 2).mean(-1, keepdim=True) + eps) * g.double()
+    ref = n @ w.double().T
+    close(G.skinny_after_chain(xg, ssq, eps, w, out_dtype=torch.float32), ref, 1e-2)
+    close(G.skinny_after_chain(xg, ssq, eps, w), ref, 1.5e-2)
+    I = N2 // 2
+    a = ref[:, :I]
+    close(G.skinny_after_chain_gated(xg, ssq, eps, w), (a * torch.sigmoid(a)) * ref[:, I:], 2e-2)
+    separate = G.skinny(K().rmsnorm(res, g, eps, torch.bfloat16), w, out_dtype=torch.float32)
+    close(G.skinny_after_chain(xg, ssq, eps, w, out_dtype=torch.float32), separate, 1e-2)
+    # row by row: a row's factor must be its own
+    got = G.skinny_after_chain(xg, ssq, eps, w, out_dtype=torch.float32).double().cpu()
+    for m in range(M):
+        assert float((got[m] - ref[m].cpu()).abs().max() / ref[m].abs().max()) < 1.5e-2
+    from gpt_fast_amd.ops.linear import HalfNormed
+    close(HalfNormed(xg, ssq, eps).materialize(), n, 1e-2)
+
+
 @pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])
 def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     from gpt_fast_amd.ops import gemm_bf16 as G
@@ -432,6 +471,21 @@ def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     close(q4, q2, 1e-2)
     close(kp4, kp2, 1e-2)
     assert torch.equal(vp4, vp2)                       # values are not rotated: same products
+    # rows whose norm arrives in two halves
+    if D % 8 == 0:
+        y = bf(torch.randn(M, 64, device=DEV))
+        wo = bf(torch.randn(D, 64, device=DEV) * 0.2)
+        res = x.clone()
+        xg, ssq = G.skinny_into_chain(y, wo, res, g)
+        kp5, vp5 = torch.zeros_like(kp), torch.zeros_like(vp)
+        q5 = G.qkv_rope_store(xg, None, 1e-5, w, freqs, tok_seq, tok_pos, table, kp5, vp5, H, G_, hd,
+                              rot, ssq=ssq)
+        kp6, vp6 = torch.zeros_like(kp), torch.zeros_like(vp)
+        q6 = G.qkv_rope_store(K().rmsnorm(res, g, 1e-5, torch.bfloat16), None, 0.0, w, freqs, tok_seq,
+                              tok_pos, table, kp6, vp6, H, G_, hd, rot)
+        close(q5, q6, 1.5e-2)
+        close(kp5, kp6, 1.5e-2)
+        close(vp5, vp6, 1.5e-2)
 
 
 def test_sampling_over_many_workgroups_equals_one_workgroup():

@@ -19,11 +19,14 @@ A new part is a class with these methods, registered under a new ``kind``; its s
 any object with that ``kind`` attribute.
 
 Optional, for speed only: a mixer or feed-forward that sets ``prepares_norm = True`` also
-takes ``then_norm=`` (the norm that reads the residual stream after it) and returns that
-norm's rows if its last kernel produced them on the way, else None; a norm offers this by
-``row_and_column_form() -> (column weights, eps)``.  A block with ``prepares_norm`` takes
-``x=`` (the rows of its first norm, ``mixer_norm``, if the caller has them) and
-``then_norm=`` and returns likewise.  Parts without the flag are called as above.
+takes ``then_norm=`` (the norm that reads the residual stream after it) and
+``takes_halves=`` and returns that norm's rows if its last kernel produced them on the way,
+else None; with ``takes_halves`` they may be an ``ops.linear.HalfNormed``, which the products
+of ``ops.linear`` accept in place of x, and a part that passes its x only to those sets
+``takes_prepared = True``.  A norm offers this by ``row_and_column_form() -> (column
+weights, eps)``.  A block with ``prepares_norm`` takes ``x=`` (the rows of its first norm,
+``mixer_norm``, if the caller has them), ``then_norm=`` and ``takes_halves=`` and returns
+likewise.  Parts without the flags are called as above and get plain tensors.
 """
 from dataclasses import dataclass
 from typing import Callable, Dict, Tuple

@@ -334,12 +334,68 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
     }
 }
 
+// The same for bfloat16 with interleaved pairs, eight elements (four pairs) per thread:
+// 16-byte loads and stores for q and k.  Needs hd and rot to be multiples of 8.
+__global__ __launch_bounds__(256) void rope_cache_bf16x8_kernel(
+        const bf16_t* __restrict__ qkv, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_pages,
+        bf16_t* __restrict__ v_pages, const float* __restrict__ freqs,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, int table_stride, int H, int Hkv, int hd, int rot) {
+    const int n = blockIdx.x;
+    const int per_head = hd / 8;
+    const int qk_chunks = (H + Hkv) * per_head, v_chunks = Hkv * per_head;
+    const int pos = tok_pos[n];
+    extern __shared__ float cs[];                          // [rot / 2][2]
+    if (blockIdx.y * 256 < qk_chunks) {
+        for (int i = threadIdx.x; i < rot / 2; i += 256)
+            sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
+        __syncthreads();
+    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= qk_chunks + v_chunks) return;
+    const int head = c / per_head, d0 = (c - head * per_head) * 8;
+    union { uint4 u; bf16_t e[8]; } in, out;
+    in.u = *(const uint4*)(qkv + ((size_t)n * (H + 2 * Hkv) + head) * hd + d0);
+    int page = 0;
+    if (k_pages && head >= H) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+    const int off = pos % GFA_PAGE;
+    if (head < H + Hkv) {
+        if (d0 < rot) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const float a = bf16_to_float(in.e[2 * p]), b = bf16_to_float(in.e[2 * p + 1]);
+                const float c_ = cs[d0 + 2 * p], s_ = cs[d0 + 2 * p + 1];
+                out.e[2 * p] = float_to_bf16(a * c_ - b * s_);
+                out.e[2 * p + 1] = float_to_bf16(b * c_ + a * s_);
+            }
+        } else {
+            out.u = in.u;
+        }
+        if (head < H) {
+            *(uint4*)(q_out + ((size_t)n * H + head) * hd + d0) = out.u;
+        } else if (k_pages) {
+            *(uint4*)(k_pages + page_row(page, head - H, off, Hkv, hd) + d0) = out.u;
+        }
+    } else if (v_pages) {
+        const int g = head - H - Hkv;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v_pages[value_elem(page, g, d0 + j, off, Hkv, hd)] = in.e[j];
+    }
+}
+
 extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages, void* v_pages,
                                     const float* freqs, const int* tok_seq, const int* tok_pos,
                                     const int* table, int table_stride, int n_tokens, int H,
                                     int Hkv, int hd, int rot, int layout, int is_bf16,
                                     hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (is_bf16 && layout == 0 && hd % 8 == 0 && rot % 8 == 0) {
+        const dim3 grid8(n_tokens, ((H + 2 * Hkv) * (hd / 8) + 255) / 256);
+        rope_cache_bf16x8_kernel<<<grid8, 256, (size_t)(rot > 0 ? rot : 2) * sizeof(float), stream>>>(
+            (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs, tok_seq,
+            tok_pos, table, table_stride, H, Hkv, hd, rot);
+        return GFA_LAUNCH_RESULT();
+    }
     const dim3 grid(n_tokens, ((H + 2 * Hkv) * (hd / 2) + 255) / 256);
     if (is_bf16)
         rope_cache_kernel<bf16_t><<<grid, 256, (size_t)rot * sizeof(float), stream>>>(

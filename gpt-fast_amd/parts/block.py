@@ -39,7 +39,8 @@ class PreNormBlock(Part):
     # Norm hand-over, optional for every part: a mixer or feed-forward that sets
     # ``prepares_norm`` takes ``then_norm=`` (the norm that reads the residual stream after
     # it) and ``takes_halves=`` (whether that norm's reader accepts an ops.linear.HalfNormed
-    # in place of x; a part says so with ``takes_prepared``), and returns that norm's rows if
+    # in place of x; a part says so with ``takes_prepared``: True, or the least number of
+    # rows from which it wants them), and returns that norm's rows if
     # it produced them on the way, else None.  A block that sets ``prepares_norm`` takes
     # ``x=`` (the rows of its first norm, if the caller has them), ``then_norm=`` and
     # ``takes_halves=`` in the same sense, and names its first norm ``mixer_norm``.
@@ -49,13 +50,19 @@ class PreNormBlock(Part):
     def takes_prepared(self):
         return getattr(self.mixer, "takes_prepared", False)
 
+    @staticmethod
+    def _wants_halves(part, n_rows: int) -> bool:
+        least = getattr(part, "takes_prepared", False)
+        return bool(least) and n_rows >= int(least)
+
     def forward(self, residual, batch, entry, x=None, then_norm=None, takes_halves=False):
         if x is None:
             x = self.mixer_norm.forward(residual)
         h = None
         if getattr(self.mixer, "prepares_norm", False):
             h = self.mixer.forward(x, batch, entry, residual, then_norm=self.feed_forward_norm,
-                                   takes_halves=getattr(self.feed_forward, "takes_prepared", False))
+                                   takes_halves=self._wants_halves(self.feed_forward,
+                                                                   residual.shape[0]))
         else:
             self.mixer.forward(x, batch, entry, residual)
         if h is None:

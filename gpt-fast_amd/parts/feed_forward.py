@@ -24,7 +24,9 @@ class GatedFeedForward(Part):
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
     prepares_norm = True
-    takes_prepared = True          # x may be an ops.linear.HalfNormed
+    # x may be an ops.linear.HalfNormed; from two rows on (the one-row gate product runs on
+    # a kernel that takes plain rows and is faster than the saving)
+    takes_prepared = 2
 
     def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
         h = L.gated_linear(x, self.w13)

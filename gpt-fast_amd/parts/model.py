@@ -81,12 +81,14 @@ class DecoderModel:
                 block.forward(residual, batch, cache.entries[n])
                 x = None
                 continue
-            takes_halves = True                    # the head is a product of ops.linear
+            # the head takes plain rows: with its many columns the halves cost more than the
+            # norm kernel they save
+            takes_halves = False
             if n + 1 < len(order):
                 nxt = self.blocks[order[n + 1].layer]
                 then_norm = getattr(nxt, "mixer_norm", None)
-                takes_halves = (getattr(nxt, "prepares_norm", False)
-                                and getattr(nxt, "takes_prepared", False))
+                least = getattr(nxt, "takes_prepared", False) if getattr(nxt, "prepares_norm", False) else False
+                takes_halves = bool(least) and residual.shape[0] >= int(least)
             else:
                 then_norm = self.final_norm if getattr(batch, "every_row_wanted", False) else None
             x = block.forward(residual, batch, cache.entries[n], x=x, then_norm=then_norm,

@@ -90,8 +90,11 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    // keys: tile kt, row kt * 16 + li of the block, dims ds * 32 + lg * 8 .. +7
-    // values: dims dt * 16 + li, keys (tile 0 | tile 1) 4 lg .. +3 of the block
+    // Row r of key tile kt stands for key 8 (r / 4) + 4 kt + r % 4 of the block, so that the
+    // eight scores a lane holds (rows 4 lg .. +3 of both tiles) belong to the eight
+    // consecutive keys 8 lg .. +7 and its value operand is one 16-byte load.
+    // keys: tile kt, row li -> that key, dims ds * 32 + lg * 8 .. +7
+    // values: dims dt * 16 + li, keys 8 lg .. +7 of the block
     auto load_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
         const int page = pages[kb >> 1];
         const int in_page = (kb & 1) * 32;
@@ -101,23 +104,21 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) {
                 const int d = ds * 32 + lg * 8;
-                kf[kt][ds].u = (d < hd) ? *(const uint4*)(kbase + (size_t)(kt * 16 + li) * hd + d)
+                kf[kt][ds].u = (d < hd) ? *(const uint4*)(kbase + (size_t)(8 * (li >> 2) + 4 * kt + (li & 3)) * hd + d)
                                         : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const int d = dt * 16 + li;
             if (d < hd) {
-                const bf16_t* vrow = v_pages + value_elem(page, g, d, in_page + lg * 4, Hkv, hd);
-                vf[dt].h[0] = *(const uint2*)vrow;
-                vf[dt].h[1] = *(const uint2*)(vrow + 16);
+                vf[dt].u = *(const uint4*)(v_pages + value_elem(page, g, d, in_page + lg * 8, Hkv, hd));
             } else {
                 vf[dt].u = make_uint4(0, 0, 0, 0);
             }
         }
     };
     auto compute_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
-        const int key0 = kb * 32 + lg * 4;
+        const int key0 = kb * 32 + lg * 8;                 // this lane's keys: key0 .. key0 + 7
         floatx4_t s[RT][2];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (key0 + (e >> 2) * 16 + (e & 3) > pmax) vf[dt].e[e] = 0;
+                    if (key0 + e > pmax) vf[dt].e[e] = 0;
         }
         // blocks wholly below every row's position (and inside every window) need no mask
         const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
                 const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const int key = key0 + (e >> 2) * 16 + (e & 3);
+                    const int key = key0 + e;
                     const float v = s[rt][e >> 2][e & 3] * scale_log2;
                     sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
                     mx = fmaxf(mx, sv[e]);
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     constexpr int DT = DS * 2, RT = TL_RT;
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
     constexpr int KPITCH = HDM * 2 + 16;                  // bytes per key row in LDS
-    constexpr int VPITCH = 64 * 2 + 8;                    // bytes per value row (one dim, 64 keys)
+    constexpr int VPITCH = 64 * 2 + 16;                   // bytes per value row (one dim, 64 keys)
     constexpr int KBYTES = 64 * KPITCH, VBYTES = HDM * VPITCH;
     extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 x (K tile, V tile)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -383,7 +384,11 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         for (int i = 0; i < K_PER; ++i) {
             const int c = threadIdx.x + i * 256;
             const int key = c / hd8, piece = c - key * hd8;
-            k_dst[i] = (FULL || c < k_chunks) ? key * KPITCH + piece * 16 : -1;
+            // keys are stored in the order the score tiles read them: within a block of 32,
+            // key 8 a + 4 t + b (a < 4, t < 2, b < 4) is row 16 t + 4 a + b, so that the
+            // eight scores of a lane belong to eight consecutive keys (as in the kernel above)
+            const int row = (key & 32) | (((key >> 2) & 1) << 4) | (((key >> 3) & 3) << 2) | (key & 3);
+            k_dst[i] = (FULL || c < k_chunks) ? row * KPITCH + piece * 16 : -1;
         }
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
@@ -426,9 +431,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
             if (v_dst[i] >= 0) {
                 Frag f;
                 f.u = vreg[i];
-                uint2* dst = (uint2*)(vt + v_dst[i]);
-                dst[0] = f.h[0];
-                dst[1] = f.h[1];
+                *(uint4*)(vt + v_dst[i]) = f.u;
             }
         }
     };
@@ -436,7 +439,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         const char* kt = smem + buf * (KBYTES + VBYTES);
         const char* vt = kt + KBYTES;
         const int in_page = (kb & 1) * 32;
-        const int key0 = kb * 32 + lg * 4;
+        const int key0 = kb * 32 + lg * 8;                 // this lane's keys: key0 .. key0 + 7
         floatx4_t s[RT][2];
 #pragma unroll
         for (int kt16 = 0; kt16 < 2; ++kt16) {
@@ -463,7 +466,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                 const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const int key = key0 + (e >> 2) * 16 + (e & 3);
+                    const int key = key0 + e;
                     sv[e] = (key <= rpos[rt] && key >= first) ? s[rt][e >> 2][e & 3] : -INFINITY;
                 }
             } else {
@@ -498,9 +501,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         for (int dt = 0; dt < DT; ++dt) {
             if (FULL || dt * 16 < hd) {
                 Frag vf;
-                const char* vrow = vt + (dt * 16 + li) * VPITCH + (in_page + lg * 4) * 2;
-                vf.h[0] = *(const uint2*)vrow;
-                vf.h[1] = *(const uint2*)(vrow + 32);
+                vf.u = *(const uint4*)(vt + (dt * 16 + li) * VPITCH + (in_page + lg * 8) * 2);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
                     o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][dt], 0, 0, 0);
@@ -560,7 +561,7 @@ static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* 
     }
     const int total = (int)(grid.x * grid.y);
     const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
-    const size_t shmem = 2 * (size_t)(64 * (HDM * 2 + 16) + HDM * (64 * 2 + 8));
+    const size_t shmem = 2 * (size_t)(64 * (HDM * 2 + 16) + HDM * (64 * 2 + 16));
     static bool raised = false;
     if (!raised) {
         hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL>,

@@ -286,3 +286,16 @@ def test_loop_with_a_session_single_token_budget():
     new, why = BatchRun(st, [[1, 2], [3]], [0, 1], max_new_tokens=1).run()
     assert new == [[7], [7]] and why == ["length", "length"]
     assert not hasattr(st, "session")                 # nothing left to decode
+
+
+def test_bench_refuses_more_than_one_gpu_in_one_line():
+    """bench.py measures one GPU: for N > 1 it prints one line that says so and exits with 2,
+    before anything touches a device."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "4"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout

@@ -285,7 +285,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
 // copied once into LDS by all four waves - each is one contiguous piece of the cache - and
 // the next page is already on its way while the current one is multiplied.  Rows of the
 // LDS tiles are padded so that the operand reads (16 rows at a time) spread over the banks.
-// The arithmetic per 32 keys is that of the kernel above.
+// The arithmetic is that of the kernel above, a page (64 keys) at a time.
 #define TL_WAVES 4
 #define TL_RT 2
 #define TL_ROWS (TL_WAVES * TL_RT * 16)
@@ -435,19 +435,20 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
             }
         }
     };
-    auto compute_block = [&](int buf, int kb) {            // kb: block of 32 keys
+    // One page (64 keys) at a time: all scores first, then the softmax of both row tiles,
+    // then the second product - long enough stretches of independent work for the matrix
+    // cores and the vector ALU to overlap inside one wave.
+    auto compute_page = [&](int buf, int pg) {
         const char* kt = smem + buf * (KBYTES + VBYTES);
         const char* vt = kt + KBYTES;
-        const int in_page = (kb & 1) * 32;
-        const int key0 = kb * 32 + lg * 8;                 // this lane's keys: key0 .. key0 + 7
-        floatx4_t s[RT][2];
+        floatx4_t s[RT][4];
 #pragma unroll
-        for (int kt16 = 0; kt16 < 2; ++kt16) {
+        for (int kt16 = 0; kt16 < 4; ++kt16) {
             Frag kf[DS];
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds)
                 kf[ds].u = (FULL || ds * 32 + lg * 8 < hd)
-                               ? *(const uint4*)(kt + (in_page + kt16 * 16 + li) * KPITCH + (ds * 32 + lg * 8) * 2)
+                               ? *(const uint4*)(kt + (kt16 * 16 + li) * KPITCH + (ds * 32 + lg * 8) * 2)
                                : make_uint4(0, 0, 0, 0);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -457,24 +458,27 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                     s[rt][kt16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ds].v, qf[rt][ds].v, s[rt][kt16], 0, 0, 0);
             }
         }
-        const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
-        Frag pf[RT];
+        const bool masked = pg * 64 + 63 > pmin || (window > 0 && pg * 64 < pmax - window + 1);
+        const int key0 = pg * 64 + lg * 8;                 // this lane's keys: key0 .. +7, key0 + 32 .. +39
+        Frag pf[RT][2];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            float sv[8];                                   // raw scores; -inf where masked
+            float sv[16];                                  // raw scores; -inf where masked
             if (masked) {
                 const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int key = key0 + e;
+                for (int e = 0; e < 16; ++e) {
+                    const int key = key0 + (e >> 3) * 32 + (e & 7);
                     sv[e] = (key <= rpos[rt] && key >= first) ? s[rt][e >> 2][e & 3] : -INFINITY;
                 }
             } else {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sv[e] = s[rt][e >> 2][e & 3];
+                for (int e = 0; e < 16; ++e) sv[e] = s[rt][e >> 2][e & 3];
             }
-            float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                             fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            float mx = fmaxf(fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                                   fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7]))),
+                             fmaxf(fmaxf(fmaxf(sv[8], sv[9]), fmaxf(sv[10], sv[11])),
+                                   fmaxf(fmaxf(sv[12], sv[13]), fmaxf(sv[14], sv[15]))));
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             mx *= scale_log2;                              // scale > 0: the order is kept
@@ -490,21 +494,24 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
             const float neg_m = (m[rt] == -INFINITY) ? 0.f : -m[rt];
             float sum = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
+            for (int e = 0; e < 16; ++e) {
                 const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], scale_log2, neg_m));
                 sum += p;
-                pf[rt].e[e] = float_to_bf16(p);
+                pf[rt][e >> 3].e[e & 7] = float_to_bf16(p);
             }
             l[rt] += sum;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             if (FULL || dt * 16 < hd) {
-                Frag vf;
-                vf.u = *(const uint4*)(vt + (dt * 16 + li) * VPITCH + (in_page + lg * 8) * 2);
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt].v, o[rt][dt], 0, 0, 0);
+                for (int hb = 0; hb < 2; ++hb) {
+                    Frag vf;
+                    vf.u = *(const uint4*)(vt + (dt * 16 + li) * VPITCH + (hb * 32 + lg * 8) * 2);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
+                }
             }
         }
     };
@@ -515,13 +522,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     for (int pg = page_lo; pg <= page_hi; ++pg) {
         const int buf = (pg - page_lo) & 1;
         if (pg < page_hi) fetch_page(pg + 1);
-        if (wave_has_rows) {
-#pragma unroll
-            for (int hb = 0; hb < 2; ++hb) {
-                const int kb = pg * 2 + hb;
-                if (kb * 32 <= pmax && kb * 32 + 31 >= w_lo) compute_block(buf, kb);
-            }
-        }
+        if (wave_has_rows && pg * 64 <= pmax && pg * 64 + 63 >= w_lo) compute_page(buf, pg);
         if (pg < page_hi) store_page(buf ^ 1, pg + 1);
         __syncthreads();
     }

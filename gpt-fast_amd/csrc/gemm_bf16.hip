@@ -242,9 +242,9 @@ struct SkinnyExtra {
     int table_stride, H, Hkv, hd, rot;
     // A norm spread over two kernels (one tile of rows).  The kernel that completes the
     // residual stream (MODE 2) also writes xg_out [M, N] = bfloat16(new residual * next_g) and
-    // ssq_out [tiles, 16]: each workgroup's share of its 16 rows' sums of squares (float, from
-    // the float residual).  The next product takes xg as its x, adds the shares in a fixed
-    // order (ssq_in [t_in, 16]) and scales its result by rsqrt(sum / K + eps): a factor per row
+    // ssq_out [tiles, share_rows]: each workgroup's share of its rows' sums of squares (float,
+    // from the float residual).  The next product takes xg as its x, adds the shares in a fixed
+    // order (ssq_in [t_in, share_rows]) and scales its result by rsqrt(sum / K + eps): a factor per row
     // commutes with the product, so this is the RMS norm of model.py:236-241.
     bf16_t* xg_out;
     const float* next_g;
@@ -252,7 +252,11 @@ struct SkinnyExtra {
     const float* ssq_in;
     int t_in;
     int share_off;            // byte offset in LDS of the waves' pieces for the shares
+    int share_rows;           // rows per share record: 4, 8 or 16 (the least that holds M)
 };
+
+// Rows per record of the sums-of-squares shares for M rows of x.
+extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
 template <int CT, int MODE, bool NORM>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
@@ -397,19 +401,23 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                     sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[pr], &rot_cs[pr]);
         }
     }
-    // second half of a two-kernel norm: lane group fg of wave w takes the shares of the
-    // column tiles fg + 4 w, + 4 NW ..., 16 rows side by side (64 contiguous bytes each).
-    // They are requested here as copies straight into a wave-private piece of LDS - no
-    // register waits for them, so nothing below is held up - and added after the product.
+    // second half of a two-kernel norm.  A share record holds R = share_rows rows side by
+    // side; one copy instruction of a wave takes 64 / R records (lane l: row l % R of record
+    // l / R), wave w takes the record groups w, w + NW, ...  The copies go straight into a
+    // wave-private piece of LDS - no register waits for them, so nothing below is held up -
+    // and are added after the product.  Every workgroup reads all shares, so their bytes
+    // count: hence the narrow records for few rows.
     constexpr int SHARES = 16;
     const bool chained = CT == 1 && ex.ssq_in != nullptr;
     float* share_lds = (float*)(smem + ex.share_off) + wave * (SHARES * 64);
+    const int R = ex.share_rows, per_copy = R ? 64 / R : 4;
     if (chained) {
 #pragma unroll
         for (int j = 0; j < SHARES; ++j) {
-            const int tile = fg + 4 * (wave + NW * j);
-            if (4 * (wave + NW * j) < ex.t_in) {          // wave-uniform
-                const float* src = ex.ssq_in + (size_t)(tile < ex.t_in ? tile : 0) * 16 + fi;
+            const int first = per_copy * (wave + NW * j);
+            if (first < ex.t_in) {                         // wave-uniform
+                const int rec = first + lane / R;
+                const float* src = ex.ssq_in + (size_t)(rec < ex.t_in ? rec : 0) * R + lane % R;
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)src,
                     (__attribute__((address_space(3))) void*)(share_lds + j * 64), 4, 0, 0);
@@ -435,20 +443,21 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             ssq[ct] += __shfl_xor(ssq[ct], 32, GFA_WAVE);
         }
     }
-    if (chained) {                                       // fixed order: lane, lane groups, waves
+    if (chained) {                                       // fixed order: lane, lanes of a row, waves
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the copies into LDS have landed
         float pre_ssq = 0.f;
 #pragma unroll
         for (int j = 0; j < SHARES; ++j) {
-            const int tile = fg + 4 * (wave + NW * j);
-            if (tile < ex.t_in) pre_ssq += share_lds[j * 64 + lane];
+            const int rec = per_copy * (wave + NW * j) + lane / R;
+            if (rec < ex.t_in) pre_ssq += share_lds[j * 64 + lane];
         }
-        for (int tile = fg + 4 * (wave + NW * SHARES); tile < ex.t_in; tile += 4 * NW)
-            pre_ssq += ex.ssq_in[(size_t)tile * 16 + fi];
-        const float other = __shfl_xor(pre_ssq, 16, GFA_WAVE);
-        pre_ssq = (fg & 1) ? other + pre_ssq : pre_ssq + other;      // (g0 + g1), (g2 + g3)
-        const float pair = __shfl_xor(pre_ssq, 32, GFA_WAVE);
-        pre_ssq = (fg & 2) ? pair + pre_ssq : pre_ssq + pair;        // (g0 + g1) + (g2 + g3)
+        for (int rec = per_copy * (wave + NW * SHARES) + lane / R; rec < ex.t_in; rec += per_copy * NW)
+            pre_ssq += ex.ssq_in[(size_t)rec * R + lane % R];
+        // lanes l, l + R, l + 2 R, ... hold parts of row l % R: a butterfly in a fixed order
+        for (int step = R; step < 64; step <<= 1) {
+            const float other = __shfl_xor(pre_ssq, step, GFA_WAVE);
+            pre_ssq = (lane & step) ? other + pre_ssq : pre_ssq + other;
+        }
         ssq[0] = pre_ssq;                                // from here on as the fused norm's sum
     }
     if (NW > 1) {
@@ -555,7 +564,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     if (MODE == 2 && ex.xg_out) {                        // this workgroup's share, rows side by side
         part_ssq += __shfl_xor(part_ssq, 16, GFA_WAVE);
         part_ssq += __shfl_xor(part_ssq, 32, GFA_WAVE);
-        if (fg == 0) ex.ssq_out[(size_t)blockIdx.x * 16 + fi] = part_ssq;
+        if (fg == 0 && fi < ex.share_rows) ex.ssq_out[(size_t)blockIdx.x * ex.share_rows + fi] = part_ssq;
     }
 }
 
@@ -678,6 +687,7 @@ extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, 
         if (M > 16 || t_in <= 0) return (int)hipErrorInvalidValue;
         ex.ssq_in = ssq_in;
         ex.t_in = t_in;
+        ex.share_rows = gfa_share_rows(M);
     }
     const int N = (H + 2 * Hkv) * hd;
     if (x_bf16)
@@ -686,8 +696,9 @@ extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, 
 }
 
 // residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
-// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [(N + 15) / 16, 16] = the
-// workgroups' shares of the rows' sums of squares.  N a multiple of 4.
+// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [(N + 15) / 16, share_rows] = the
+// workgroups' shares of the rows' sums of squares; share_rows = gfa_share_rows(M).  N a
+// multiple of 4.
 extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* residual, int M,
                                           int N, int K, const float* next_g, void* xg_out,
                                           float* ssq_out, hipStream_t stream) {
@@ -695,6 +706,7 @@ extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* r
     if (M > 16 || K <= 0 || K % 8 != 0 || N % 4 != 0 || !next_g || !xg_out || !ssq_out)
         return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
+    ex.share_rows = gfa_share_rows(M);
     ex.next_g = next_g;
     ex.xg_out = (bf16_t*)xg_out;
     ex.ssq_out = ssq_out;
@@ -702,7 +714,8 @@ extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* r
 }
 
 // The product that follows: x = xg [M <= 16, K], the result scaled by
-// rsqrt(sum of ssq_in[:, m] / K + eps).  mode 0 bfloat16 out, 1 float out, 3 gate.
+// rsqrt(sum of ssq_in[:, m] / K + eps), ssq_in [t_in, gfa_share_rows(M)].  mode 0 bfloat16
+// out, 1 float out, 3 gate.
 extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, int t_in, float eps,
                                            const void* w, void* out, int M, int N, int K, int ldo,
                                            int mode, int gate_rows, hipStream_t stream) {
@@ -711,6 +724,7 @@ extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, 
     SkinnyExtra ex = {};
     ex.ssq_in = ssq_in;
     ex.t_in = t_in;
+    ex.share_rows = gfa_share_rows(M);
     ex.eps = eps;
     const bf16_t* xp = (const bf16_t*)xg;
     const bf16_t* wp = (const bf16_t*)w;

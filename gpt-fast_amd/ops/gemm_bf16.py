@@ -79,11 +79,17 @@ def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:
     return 0 < n_rows <= 16 and n_out % 8 == 0 and inner % 8 == 0
 
 
+def share_rows(n_rows: int) -> int:
+    """Rows per record of the sums-of-squares shares for this many rows of x."""
+    return 4 if n_rows <= 4 else 8 if n_rows <= 8 else 16
+
+
 def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
                       next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
-    ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, 16]: per
-    workgroup (16 columns) its share of each row's sum of squares.  Up to 16 rows."""
+    ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, R]: per
+    workgroup (16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
+    record (the least that holds M).  Up to 16 rows."""
     _check_operands(x, w, "skinny_into_chain")
     M, K = x.shape
     N = w.shape[0]
@@ -95,7 +101,7 @@ def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
     if not can_chain_norm(M, N, K):
         raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
     xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    ssq = torch.empty(((N + 15) // 16, 16), dtype=torch.float32, device=x.device)
+    ssq = torch.empty(((N + 15) // 16, share_rows(M)), dtype=torch.float32, device=x.device)
     check(library("gemm_bf16").gfa_skinny_into_chain_bf16(
         ptr(x), ptr(w), ptr(residual), _i(M), _i(N), _i(K), ptr(next_g), ptr(xg), ptr(ssq),
         stream_handle()), "skinny_into_chain")
@@ -107,8 +113,9 @@ def _check_chain(xg, ssq, w, what):
     require_device(ssq)
     if xg.shape[0] > 16 or w.shape[1] % 8:
         raise KernelError(f"{what}: takes 1..16 rows and an inner size that is a multiple of 8")
-    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[1] != 16 or not ssq.is_contiguous():
-        raise KernelError(f"{what}: ssq must be contiguous float32 [shares, 16]")
+    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[1] != share_rows(xg.shape[0]) \
+            or not ssq.is_contiguous():
+        raise KernelError(f"{what}: ssq must be contiguous float32 [shares, {share_rows(xg.shape[0])}]")
 
 
 def skinny_after_chain(xg, ssq, eps: float, w, out_dtype=torch.bfloat16):

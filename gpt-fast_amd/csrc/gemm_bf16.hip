@@ -575,9 +575,11 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     const int tiles = (N + 15) / 16;
     const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
     const int ct = (M + 15) / 16;
-    int nw = 1;                                          // waves per tile: aim at >= 2048 waves
+    int nw = 1;                                          // waves per tile: aim at >= 2048 waves,
     const int nw_max = (MODE == 3) ? 4 : 8;
-    while (nw < nw_max && tiles * nw < 2048 && pieces >= 4 * nw) nw *= 2;
+    // at least four waves per tile where K allows: one wave walking sixteen rows alone
+    // streams measurably slower than four that share them
+    while (nw < nw_max && (tiles * nw < 2048 || nw < 4) && pieces >= 4 * nw) nw *= 2;
     size_t shmem = (size_t)nw * RT * SM_TILE;
     const size_t red = (size_t)nw * RT * ct * 64 * sizeof(floatx4_t) + (size_t)nw * ct * 16 * sizeof(float);
     if (nw > 1 && red > shmem) shmem = red;

@@ -224,11 +224,7 @@ union Frag8 {
 
 // What the fused variants need beside the product itself.
 struct SkinnyExtra {
-    // NORM: x is the float residual stream; the product takes x * norm_w rounded to
-    // bfloat16 and is scaled by rsqrt(mean(x^2) + eps) at the end (model.py:236-241)
-    const float* x_f32;
-    const float* norm_w;
-    float eps;
+    float eps;                // of the norm whose row factor this product applies (below)
     // MODE 4: the columns are q heads, k heads, v heads (model.py:195-199); q and k pairs
     // (2i, 2i+1) are rotated by tok_pos * freqs[i] (model.py:281-293), q goes to q_out
     // [M, H, hd], k and v into the pages (model.py:91-100) unless k_pages is null
@@ -258,7 +254,7 @@ struct SkinnyExtra {
 // Rows per record of the sums-of-squares shares for M rows of x.
 extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-template <int CT, int MODE, bool NORM>
+template <int CT, int MODE>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, SkinnyExtra ex) {
@@ -312,20 +308,11 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     // loads return in order, so waiting for x must not mean waiting for the prefetch.
     constexpr int XS = SM_SUBK / 32;
     uint4 xraw[XS][CT];                                  // bfloat16 x, or converted below
-    float4 xf0[NORM ? XS : 1], xf1[NORM ? XS : 1], xg0[NORM ? XS : 1], xg1[NORM ? XS : 1];
     auto load_x = [&](int t) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
-            if (NORM) {                                  // CT == 1
-                const bool ok = fi < M && kk < K;
-                const float* xr = ex.x_f32 + (size_t)(ok ? fi : 0) * K + (ok ? kk : 0);
-                const float* gr = ex.norm_w + (ok ? kk : 0);
-                xf0[s] = *(const float4*)xr;
-                xf1[s] = *(const float4*)(xr + 4);
-                xg0[s] = *(const float4*)gr;
-                xg1[s] = *(const float4*)(gr + 4);
-            } else {
+            {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     const int m = ct * 16 + fi;
@@ -339,24 +326,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             Frag8 b[CT];
-            if (NORM) {
-                const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
-                if (fi < M && kk < K) {
-                    const float4 a0 = xf0[s], a1 = xf1[s], g0 = xg0[s], g1 = xg1[s];
-                    ssq[0] += a0.x * a0.x + a0.y * a0.y + a0.z * a0.z + a0.w * a0.w +
-                              a1.x * a1.x + a1.y * a1.y + a1.z * a1.z + a1.w * a1.w;
-                    bf16_t* e = (bf16_t*)&b[0].u;
-                    e[0] = float_to_bf16(a0.x * g0.x); e[1] = float_to_bf16(a0.y * g0.y);
-                    e[2] = float_to_bf16(a0.z * g0.z); e[3] = float_to_bf16(a0.w * g0.w);
-                    e[4] = float_to_bf16(a1.x * g1.x); e[5] = float_to_bf16(a1.y * g1.y);
-                    e[6] = float_to_bf16(a1.z * g1.z); e[7] = float_to_bf16(a1.w * g1.w);
-                } else {
-                    b[0].u = make_uint4(0, 0, 0, 0);
-                }
-            } else {
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s][ct];
-            }
+            for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s][ct];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 Frag8 a;
@@ -436,13 +407,6 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             multiply_piece(t + 1);
         }
     }
-    if (NORM) {                                          // this wave's share of sum x^2 of row fi
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            ssq[ct] += __shfl_xor(ssq[ct], 16, GFA_WAVE);
-            ssq[ct] += __shfl_xor(ssq[ct], 32, GFA_WAVE);
-        }
-    }
     if (chained) {                                       // fixed order: lane, lanes of a row, waves
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the copies into LDS have landed
         float pre_ssq = 0.f;
@@ -458,7 +422,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             const float other = __shfl_xor(pre_ssq, step, GFA_WAVE);
             pre_ssq = (lane & step) ? other + pre_ssq : pre_ssq + other;
         }
-        ssq[0] = pre_ssq;                                // from here on as the fused norm's sum
+        ssq[0] = pre_ssq;                                // this wave's part of the row's sum
     }
     if (NW > 1) {
         __syncthreads();                                 // staging is done; reuse it for the sums
@@ -468,7 +432,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) red[((wave * RT + rt) * CT + ct) * 64 + lane] = acc[rt][ct];
-        if ((NORM || chained) && fg == 0) {
+        if (chained && fg == 0) {
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) red_s[(wave * CT + ct) * 16 + fi] = ssq[ct];
         }
@@ -479,7 +443,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += red[((wv * RT + rt) * CT + ct) * 64 + lane];
-            if (NORM || chained) {
+            if (chained) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) ssq[ct] += red_s[(wv * CT + ct) * 16 + fi];
             }
@@ -490,7 +454,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     for (int ct = 0; ct < CT; ++ct) {
         const int m = ct * 16 + fi;
         if (m >= M) continue;
-        if (NORM || chained) {
+        if (chained) {
             const float rs = rsqrtf(ssq[ct] / (float)K + ex.eps);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) acc[rt][ct] *= rs;
@@ -568,7 +532,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     }
 }
 
-template <int MODE, bool NORM>
+template <int MODE>
 static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
                               int ldo, int gate_rows, const SkinnyExtra& ex, hipStream_t stream) {
     constexpr int RT = (MODE == 3) ? 2 : 1;
@@ -598,22 +562,17 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     do {                                                                                          \
         static bool raised = false;                                                               \
         if (!raised) {                                                                            \
-            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, NORM>,                 \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE>,                 \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, NORM><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
+        skinny_mfma_kernel<CTV, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
     } while (0)
-    if (NORM) {                                          // the fused norm serves one 16-row tile
-        if (ct != 1) return (int)hipErrorInvalidValue;
-        GFA_LAUNCH_MFMA(1);
-    } else {
-        switch (ct) {
-            case 1: GFA_LAUNCH_MFMA(1); break;
-            case 2: GFA_LAUNCH_MFMA((NORM ? 1 : 2)); break;
-            case 3: GFA_LAUNCH_MFMA((NORM ? 1 : 3)); break;
-            default: GFA_LAUNCH_MFMA((NORM ? 1 : 4)); break;
-        }
+    switch (ct) {
+        case 1: GFA_LAUNCH_MFMA(1); break;
+        case 2: GFA_LAUNCH_MFMA(2); break;
+        case 3: GFA_LAUNCH_MFMA(3); break;
+        default: GFA_LAUNCH_MFMA(4); break;
     }
 #undef GFA_LAUNCH_MFMA
     return GFA_LAUNCH_RESULT();
@@ -627,52 +586,27 @@ extern "C" int gfa_skinny_mfma_bf16(const void* x, const void* w, void* out, int
     const bf16_t* wp = (const bf16_t*)w;
     SkinnyExtra ex = {};
     switch (mode) {
-        case 0: return launch_skinny_mfma<0, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 1: return launch_skinny_mfma<1, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 2: return launch_skinny_mfma<2, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 3: return launch_skinny_mfma<3, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 0: return launch_skinny_mfma<0>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 1: return launch_skinny_mfma<1>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 2: return launch_skinny_mfma<2>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 3: return launch_skinny_mfma<3>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
     }
     return (int)hipErrorInvalidValue;
 }
 
-// The same products reading the float residual stream through an RMS norm
-// (x_f32 [M, K], norm_w [K]): modes 0, 1 and 3 as above.
-extern "C" int gfa_skinny_norm_bf16(const float* x_f32, const float* norm_w, float eps, const void* w,
-                                    void* out, int M, int N, int K, int ldo, int mode,
-                                    int gate_rows, hipStream_t stream) {
-    if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 8 != 0) return (int)hipErrorInvalidValue;
-    const bf16_t* wp = (const bf16_t*)w;
-    SkinnyExtra ex = {};
-    ex.x_f32 = x_f32;
-    ex.norm_w = norm_w;
-    ex.eps = eps;
-    switch (mode) {
-        case 0: return launch_skinny_mfma<0, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 1: return launch_skinny_mfma<1, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 3: return launch_skinny_mfma<3, true>(nullptr, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-    }
-    return (int)hipErrorInvalidValue;
-}
-
-// norm -> fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
+// Fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
 // w [(H + 2 Hkv) hd, K]; head size a multiple of 16, rotary width even, interleaved pairs.
-// Either x_f32 with its norm (x_bf16 null), or x_bf16 already normed (up to 64 rows), or
-// x_bf16 with ssq_in [t_in, 16]: the two halves of a norm that gfa_skinny_into_chain_bf16
-// left (eps the norm's; up to 16 rows).
-extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, float eps,
-                                       const void* x_bf16, const float* ssq_in, int t_in,
+// x [M <= 64, K] are normed rows; or, with ssq_in [t_in, gfa_share_rows(M)], the two halves of
+// a norm that gfa_skinny_into_chain_bf16 left (eps the norm's; up to 16 rows).
+extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t_in, float eps,
                                        const void* w, void* q_out, void* k_pages, void* v_pages,
                                        const float* freqs, const int* tok_seq, const int* tok_pos,
                                        const int* table, int table_stride, int M, int K, int H,
                                        int Hkv, int hd, int rot, hipStream_t stream) {
     if (M <= 0) return 0;
-    if (M > (x_bf16 ? 64 : 16) || K <= 0 || K % 8 != 0 || hd % 16 != 0 || rot % 2 != 0 || rot > hd)
+    if (M > 64 || K <= 0 || K % 8 != 0 || hd % 16 != 0 || rot % 2 != 0 || rot > hd)
         return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
-    ex.x_f32 = x_f32;
-    ex.norm_w = norm_w;
-    ex.eps = eps;
     ex.q_out = (bf16_t*)q_out;
     ex.k_pages = (bf16_t*)k_pages;
     ex.v_pages = (bf16_t*)v_pages;
@@ -685,16 +619,15 @@ extern "C" int gfa_qkv_rope_store_bf16(const float* x_f32, const float* norm_w, 
     ex.Hkv = Hkv;
     ex.hd = hd;
     ex.rot = rot;
-    if (x_bf16 && ssq_in) {                               // second half of a two-kernel norm
+    if (ssq_in) {                                         // second half of a two-kernel norm
         if (M > 16 || t_in <= 0) return (int)hipErrorInvalidValue;
         ex.ssq_in = ssq_in;
         ex.t_in = t_in;
         ex.share_rows = gfa_share_rows(M);
+        ex.eps = eps;
     }
     const int N = (H + 2 * Hkv) * hd;
-    if (x_bf16)
-        return launch_skinny_mfma<4, false>((const bf16_t*)x_bf16, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
-    return launch_skinny_mfma<4, true>(nullptr, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
+    return launch_skinny_mfma<4>((const bf16_t*)x, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
 }
 
 // residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
@@ -712,7 +645,7 @@ extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* r
     ex.next_g = next_g;
     ex.xg_out = (bf16_t*)xg_out;
     ex.ssq_out = ssq_out;
-    return launch_skinny_mfma<2, false>((const bf16_t*)x, (const bf16_t*)w, residual, M, N, K, N, 0, ex, stream);
+    return launch_skinny_mfma<2>((const bf16_t*)x, (const bf16_t*)w, residual, M, N, K, N, 0, ex, stream);
 }
 
 // The product that follows: x = xg [M <= 16, K], the result scaled by
@@ -731,9 +664,9 @@ extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, 
     const bf16_t* xp = (const bf16_t*)xg;
     const bf16_t* wp = (const bf16_t*)w;
     switch (mode) {
-        case 0: return launch_skinny_mfma<0, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 1: return launch_skinny_mfma<1, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
-        case 3: return launch_skinny_mfma<3, false>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 0: return launch_skinny_mfma<0>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 1: return launch_skinny_mfma<1>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 3: return launch_skinny_mfma<3>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
     }
     return (int)hipErrorInvalidValue;
 }

@@ -163,65 +163,14 @@ def wide_f32_out(x: torch.Tensor, w: torch.Tensor):
         return out
 
 
-def _check_normed(x_f32, norm_w, w, what):
-    require_device(x_f32, norm_w, w)
-    require_contiguous(x=x_f32, norm_w=norm_w, w=w)
-    if x_f32.dtype != torch.float32 or norm_w.dtype != torch.float32 or w.dtype != torch.bfloat16:
-        raise KernelError(f"{what}: x and the norm weight must be float32, w bfloat16")
-    if x_f32.dim() != 2 or w.dim() != 2 or x_f32.shape[1] != w.shape[1] \
-            or norm_w.numel() != w.shape[1]:
-        raise KernelError(f"{what}: x {tuple(x_f32.shape)}, norm {tuple(norm_w.shape)} and "
-                          f"w {tuple(w.shape)} do not fit")
-    if not 0 < x_f32.shape[0] <= 16 or w.shape[1] % 8:
-        raise KernelError(f"{what}: takes 1..16 rows and an inner size that is a multiple of 8")
-
-
-def can_fuse_norm(n_rows: int, inner: int) -> bool:
-    # beyond one 16-row tile the float32 reads of x outweigh the saved norm kernel
-    return 0 < n_rows <= 16 and inner % 8 == 0
-
-
-def skinny_normed(x_f32, norm_w, eps: float, w, out_dtype=torch.bfloat16):
-    """rmsnorm(x_f32; norm_w, eps) times w transposed, one kernel: [M, N] in out_dtype."""
-    _check_normed(x_f32, norm_w, w, "skinny_normed")
-    M, K = x_f32.shape
-    N = w.shape[0]
-    if out_dtype not in (torch.bfloat16, torch.float32):
-        raise KernelError(f"skinny_normed: output type {out_dtype}")
-    out = torch.empty((M, N), dtype=out_dtype, device=w.device)
-    check(library("gemm_bf16").gfa_skinny_norm_bf16(
-        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(w), ptr(out), _i(M), _i(N), _i(K), _i(N),
-        _i(0 if out_dtype == torch.bfloat16 else 1), _i(0), stream_handle()), "skinny_normed")
-    return out
-
-
-def skinny_normed_gated(x_f32, norm_w, eps: float, w13):
-    """silu(n W1^T) * (n W3^T) with n = rmsnorm(x_f32), one kernel: bfloat16 [M, I]."""
-    _check_normed(x_f32, norm_w, w13, "skinny_normed_gated")
-    M, K = x_f32.shape
-    if w13.shape[0] % 2:
-        raise KernelError("skinny_normed_gated: w13 needs an even number of rows")
-    I = w13.shape[0] // 2
-    out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
-    check(library("gemm_bf16").gfa_skinny_norm_bf16(
-        ptr(x_f32), ptr(norm_w), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I), _i(K),
-        _i(I), _i(3), _i(I), stream_handle()), "skinny_normed_gated")
-    return out
-
-
-def qkv_rope_store(x, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, k_pages,
-                   v_pages, n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int,
-                   ssq: Optional[torch.Tensor] = None):
+def qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages, n_heads: int,
+                   n_kv_heads: int, head_dim: int, rotary_dim: int,
+                   ssq: Optional[torch.Tensor] = None, eps: float = 0.0):
     """Fused q/k/v projection, rotation of interleaved pairs and the cache write in one
-    kernel; returns q [M, H, hd].  ``x`` is either the float32 residual stream, read
-    through the RMS norm (``norm_w``, ``eps``; up to 16 rows), or bfloat16 rows that are
-    normed already (``norm_w`` None; up to 64 rows), or with ``ssq`` the two halves of a
-    norm as :func:`skinny_into_chain` leaves them (``eps`` the norm's; up to 16 rows).
-    k_pages None: nothing is stored."""
-    fused_norm = x.dtype == torch.float32
-    if fused_norm:
-        _check_normed(x, norm_w, wqkv, "qkv_rope_store")
-    elif ssq is not None:
+    kernel; returns q [M, H, hd].  ``x`` [M, K] bfloat16 holds normed rows (up to 64), or,
+    with ``ssq`` and ``eps``, the two halves of a norm as :func:`skinny_into_chain` leaves
+    them (up to 16 rows).  k_pages None: nothing is stored."""
+    if ssq is not None:
         _check_chain(x, ssq, wqkv, "qkv_rope_store")
     else:
         _check_operands(x, wqkv, "qkv_rope_store")
@@ -251,9 +200,7 @@ def qkv_rope_store(x, norm_w, eps: float, wqkv, freqs, tok_seq, tok_pos, table, 
             raise KernelError("qkv_rope_store: pages have the wrong shape or dtype")
     q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=wqkv.device)
     check(library("gemm_bf16").gfa_qkv_rope_store_bf16(
-        ptr(x if fused_norm else None), ptr(norm_w if fused_norm else None),
-        ctypes.c_float(eps if fused_norm or ssq is not None else 0.0),
-        ptr(None if fused_norm else x), ptr(ssq), _i(0 if ssq is None else ssq.shape[0]), ptr(wqkv),
+        ptr(x), ptr(ssq), _i(0 if ssq is None else ssq.shape[0]), ctypes.c_float(eps), ptr(wqkv),
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table),
         _i(table.shape[1]), _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim),
         _i(rotary_dim), stream_handle()), "qkv_rope_store")

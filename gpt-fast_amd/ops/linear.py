@@ -139,12 +139,12 @@ def can_project_rotate_store(x: torch.Tensor, wqkv: torch.Tensor, head_dim: int)
             and wqkv.shape[1] % 8 == 0 and head_dim % 16 == 0)
 
 
-def qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
-                   n_heads, n_kv_heads, head_dim, rotary_dim):
-    if isinstance(residual, HalfNormed):
-        h = residual
-        return _fast().qkv_rope_store(h.xg, None, h.eps, wqkv, freqs, tok_seq, tok_pos, table,
-                                      k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotary_dim,
-                                      ssq=h.ssq)
-    return _fast().qkv_rope_store(residual, norm_w, eps, wqkv, freqs, tok_seq, tok_pos, table,
-                                  k_pages, v_pages, n_heads, n_kv_heads, head_dim, rotary_dim)
+def qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages, n_heads, n_kv_heads,
+                   head_dim, rotary_dim):
+    """q [M, H, hd] of normed rows ``x`` (a tensor or a :class:`HalfNormed`) through the fused
+    projection / rotation / cache-write kernel."""
+    if isinstance(x, HalfNormed):
+        return _fast().qkv_rope_store(x.xg, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
+                                      n_heads, n_kv_heads, head_dim, rotary_dim, ssq=x.ssq, eps=x.eps)
+    return _fast().qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
+                                  n_heads, n_kv_heads, head_dim, rotary_dim)

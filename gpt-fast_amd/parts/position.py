@@ -78,7 +78,7 @@ class RotaryPosition(Part):
             return None
         write = entry is not None and entry.writes
         return L.qkv_rope_store(
-            x, None, 0.0, wqkv, self.freqs, batch.tok_seq, batch.tok_pos,
+            x, wqkv, self.freqs, batch.tok_seq, batch.tok_pos,
             batch.table(entry.group_id), entry.k_pages if write else None,
             entry.v_pages if write else None, n_heads, n_kv_heads, head_dim, self.spec.rotary_dim)
 

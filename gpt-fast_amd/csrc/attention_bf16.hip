@@ -36,7 +36,7 @@ union Frag {
 #define LOG2E 1.4426950408889634f
 
 template <int DS, int RT, bool PREFETCH>
-__global__ __launch_bounds__(256) void attention_mfma_kernel(
+__global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
@@ -215,17 +215,17 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
         lt[rt] += __shfl_xor(lt[rt], 32, 64);
     }
     if (nw > 1) {                 // the waves' partial results meet in LDS, added in wave order
-        float* sm_ml = (float*)smem;                                  // [nw][RT][16][2]
-        floatx4_t* sm_o = (floatx4_t*)(smem + (size_t)nw * RT * 16 * 2 * sizeof(float));
+        float* sm_ml = (float*)smem;                                  // [nw - 1][RT][16][2]: waves 1 ..
+        floatx4_t* sm_o = (floatx4_t*)(smem + (size_t)(nw - 1) * RT * 16 * 2 * sizeof(float));
         if (wave > 0) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 if (lg == 0) {
-                    sm_ml[((wave * RT + rt) * 16 + li) * 2] = m[rt];
-                    sm_ml[((wave * RT + rt) * 16 + li) * 2 + 1] = lt[rt];
+                    sm_ml[(((wave - 1) * RT + rt) * 16 + li) * 2] = m[rt];
+                    sm_ml[(((wave - 1) * RT + rt) * 16 + li) * 2 + 1] = lt[rt];
                 }
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) sm_o[((wave * RT + rt) * DT + dt) * 64 + lane] = o[rt][dt];
+                for (int dt = 0; dt < DT; ++dt) sm_o[(((wave - 1) * RT + rt) * DT + dt) * 64 + lane] = o[rt][dt];
             }
         }
         __syncthreads();
@@ -233,9 +233,9 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
         for (int w = 1; w < nw; ++w)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const float mw = sm_ml[((w * RT + rt) * 16 + li) * 2];
+                const float mw = sm_ml[(((w - 1) * RT + rt) * 16 + li) * 2];
                 if (mw == -INFINITY) continue;
-                const float lw = sm_ml[((w * RT + rt) * 16 + li) * 2 + 1];
+                const float lw = sm_ml[(((w - 1) * RT + rt) * 16 + li) * 2 + 1];
                 const float m_new = fmaxf(m[rt], mw);
                 const float a = __builtin_amdgcn_exp2f(m[rt] - m_new);     // 0 if this wave saw no key
                 const float b = __builtin_amdgcn_exp2f(mw - m_new);
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
                 m[rt] = m_new;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
-                    o[rt][dt] = o[rt][dt] * a + sm_o[((w * RT + rt) * DT + dt) * 64 + lane] * b;
+                    o[rt][dt] = o[rt][dt] * a + sm_o[(((w - 1) * RT + rt) * DT + dt) * 64 + lane] * b;
             }
     }
 
@@ -617,7 +617,7 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
                              const int* start_pos, const int* table, int table_stride, bf16_t* out,
                              float* ws_o, float* ws_ml, int H, int Hkv, int hd, float sl2, int window,
                              int n_splits, int total_rows) {
-    const size_t shmem = nw > 1 ? (size_t)nw * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
+    const size_t shmem = nw > 1 ? (size_t)(nw - 1) * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
     if (rt == 1)
         attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     else if (rt == 2)
@@ -628,7 +628,7 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
 
 // q, out [n_tokens, H, hd]; the sequences' token runs are given by q_start [n_seqs + 1] and
 // their first positions by start_pos [n_seqs].  rt (1, 2 or 4) 16-row tiles per wave;
-// n_waves (1..4) waves per workgroup share the key blocks of their rows;
+// n_waves (1..4; up to 8 with rt 1) waves per workgroup share the key blocks of their rows;
 // max_tiles = most waves any sequence needs per kv head.  With n_splits > 1, ws_o
 // [n_splits, n_tokens * H, hd] and ws_ml [n_splits, n_tokens * H, 2] hold the partials.
 extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void* v_pages,
@@ -640,8 +640,8 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || max_tiles < 1 ||
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
-        (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > 4 ||
-        (size_t)n_waves * rt * (128 + (hd <= 64 ? 2 : hd <= 128 ? 4 : 8) * 2 * 1024) > 65536)
+        (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > (rt == 1 ? 8 : 4) ||
+        (size_t)(n_waves - 1) * rt * (128 + (hd <= 64 ? 2 : hd <= 128 ? 4 : 8) * 2 * 1024) > 65536)
         return (int)hipErrorInvalidValue;
     const dim3 grid(max_tiles, Hkv, n_seqs * n_splits);
     const float sl2 = scale * LOG2E;

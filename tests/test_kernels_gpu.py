@@ -282,6 +282,50 @@ def test_attention_finds_one_far_key():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_query", [1, 40])
+def test_attention_window_edge(dtype, n_query):
+    """A window of W keys: the key at distance W - 1 is the last one inside, the key at
+    distance W the first one outside.  Two keys are made to stand out, one on each side of
+    the edge of the last query: the output must be the inner one's value; with the outer
+    one alone in sight of the score, it must not show.  One query row (the decode kernel)
+    and forty (the prompt kernel)."""
+    from gpt_fast_amd.ops import attention as A
+    H, G, hd, S, W = 4, 2, 64, 333, 70
+    for inside in (True, False):
+        k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=17)
+        last = S - 1
+        edge_in, edge_out = last - W + 1, last - W
+        target = edge_in if inside else edge_out
+        q = torch.randn(n_query, H, hd) * 0.01
+        for h in range(H):
+            q[-1, h] = ks[0][target, h // 2].float() * 40.0
+        q = q.to(dtype)
+
+        class B:
+            pass
+        batch = B()
+        pos = list(range(S - n_query, S))
+        batch.tok_seq = torch.zeros(n_query, dtype=torch.int32, device=DEV)
+        batch.tok_pos = torch.tensor(pos, dtype=torch.int32, device=DEV)
+        batch.n_tokens, batch.n_seqs = n_query, 1
+        batch.max_q_len, batch.max_kv_len, batch.is_decode = n_query, S, n_query == 1
+        batch.q_start = torch.tensor([0, n_query], dtype=torch.int32, device=DEV)
+        batch.start_pos = torch.tensor([S - n_query], dtype=torch.int32, device=DEV)
+        batch.host_q_start, batch.host_start_pos = [0, n_query], [S - n_query]
+        out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, 1.0, W).cpu().float()
+        for h in range(H):
+            g = h // 2
+            if inside:
+                close(out[-1, h], vs[0][target, g].float(), 2e-2)
+            else:
+                # the outer key is masked: the row is an ordinary softmax over the window
+                kk = ks[0][edge_in:last + 1, g].float()
+                p = torch.softmax(kk @ q[-1, h].float(), 0)
+                close(out[-1, h], p @ vs[0][edge_in:last + 1, g].float(), 3e-2)
+                assert float((out[-1, h] - vs[0][target, g].float()).abs().max()) > 0.1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("layout", [0, 1])
 @pytest.mark.parametrize("H,G,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 2, 128, 128)])
 def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):

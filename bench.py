@@ -104,6 +104,7 @@ def main():
     ap.add_argument("--preset", default="llama-3.1-8b",
                     help="shape to run (headline: llama-3.1-8b; others: 7B, llama-3.1-70b, ...)")
     ap.add_argument("--prompt-len", type=int, default=128)
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the timed prompt")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
     args = ap.parse_args()
@@ -163,7 +164,7 @@ def main():
                      "frac": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        T = 2048
+        T = args.prefill_tokens
         pt = prefill_run(engine, T)
         flops = prefill_flops(cfg, cfg.num_hidden_layers, T)
         out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),

@@ -9,8 +9,13 @@ _i = ctypes.c_int
 _f = ctypes.c_float
 
 TARGET_WAVES = 1024        # single-token steps split the context until this many waves run
-MIN_KEYS_PER_SPLIT = 128
 MAX_SPLITS = 16
+# A wave takes its keys one 32-key block after another, each a round trip to memory, and the
+# splits are summed by a second kernel whose cost grows with them: up to FEW_SPLITS a wave may
+# be left with 64 keys, beyond that with 128 (measured at contexts of 256 to 4096 keys).
+FEW_SPLITS = 4
+KEYS_PER_WAVE_FEW = 64
+KEYS_PER_WAVE_MANY = 128
 
 
 TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
@@ -27,8 +32,10 @@ def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int)
         nw = 4 if hd <= 128 else 2
         tiles = (R + 15) // 16
         waves = n_seqs * G * tiles * nw
-        splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS,
-                     max(1, table_width * 64 // (MIN_KEYS_PER_SPLIT * nw)))
+        keys = table_width * 64
+        by_keys = max(min(FEW_SPLITS, keys // (KEYS_PER_WAVE_FEW * nw)),
+                      keys // (KEYS_PER_WAVE_MANY * nw))
+        splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS, by_keys)
         return rt, nw, tiles, max(splits, 1)
     rt = PREFILL_ROW_TILES if hd <= 128 else min(PREFILL_ROW_TILES, 2)
     rows = max_q_len * R

@@ -94,6 +94,50 @@ def llama_bindings(c: LlamaConfig) -> CheckpointLayout:
     return CheckpointLayout(tuple(b), ignored=(r"\.rotary_emb\.inv_freq$",))
 
 
+def llama_native_layouts(c: LlamaConfig):
+    """The reference's own tensor names, as its state dict has them after conversion
+    (model.py:107-110, 158-159, 172-175, 222-224): rows already interleaved, the three
+    projections fused as ``wqkv`` - or still apart as ``wq``, ``wk``, ``wv``, which the
+    reference joins without a permutation when it loads (model.py:184-189)."""
+    D, H, G, hd = c.hidden_size, c.num_attention_heads, c.num_key_value_heads, c.head_dim
+    I, V = c.intermediate_size, c.vocab_size
+
+    def layout(fused: bool) -> CheckpointLayout:
+        b = [Binding("tok_embeddings.weight", (Source("tok_embeddings.weight", (V, D)),))]
+        for i in range(c.num_hidden_layers):
+            p = f"layers.{i}."
+            if fused:
+                qkv = Binding(p + "attention.wqkv",
+                              (Source(p + "attention.wqkv.weight", ((H + 2 * G) * hd, D)),))
+            else:
+                qkv = Binding(p + "attention.wqkv",
+                              (Source(p + "attention.wq.weight", (H * hd, D)),
+                               Source(p + "attention.wk.weight", (G * hd, D)),
+                               Source(p + "attention.wv.weight", (G * hd, D))),
+                              combine=torch.cat)
+            b += [
+                Binding(p + "attention_norm.weight",
+                        (Source(p + "attention_norm.weight", (D,), "norm"),), role="vector"),
+                qkv,
+                Binding(p + "attention.wo", (Source(p + "attention.wo.weight", (D, H * hd)),)),
+                Binding(p + "ffn_norm.weight",
+                        (Source(p + "ffn_norm.weight", (D,), "norm"),), role="vector"),
+                Binding(p + "feed_forward.w13",
+                        (Source(p + "feed_forward.w1.weight", (I, D)),
+                         Source(p + "feed_forward.w3.weight", (I, D))),
+                        combine=torch.cat),
+                Binding(p + "feed_forward.w2", (Source(p + "feed_forward.w2.weight", (D, I)),)),
+            ]
+        b.append(Binding("norm.weight", (Source("norm.weight", (D,), "norm"),), role="vector"))
+        b.append(Binding("output.weight", (Source("output.weight", (V, D)),),
+                         alias_of="tok_embeddings.weight" if c.tie_word_embeddings else None))
+        # buffers of a run that a saved state dict may carry (model.py:87-89, 133-134)
+        return CheckpointLayout(tuple(b), ignored=(r"\.kv_cache\.", r"^freqs_cis$",
+                                                   r"^causal_mask$", r"^rope\.freqs$"))
+
+    return (layout(True), layout(False))
+
+
 LLAMA = register_architecture(Architecture(
     names=("LlamaForCausalLM", "llama"),
     read_config=LlamaConfig.from_dict,
@@ -101,4 +145,5 @@ LLAMA = register_architecture(Architecture(
     bindings=llama_bindings,
     config_dict=LlamaConfig.to_dict,
     presets=LlamaConfig.from_name,
+    other_layouts=llama_native_layouts,
 ))

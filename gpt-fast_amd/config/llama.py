@@ -81,7 +81,14 @@ class LlamaConfig:
         if act != "silu":
             raise ConfigError(f"hidden_act='{act}': only 'silu' (reference model.py:227)")
 
+        # newer folders keep the base and the scaling rule together under "rope_parameters"
+        together = c.get("rope_parameters")
+        if not isinstance(together, dict):
+            together = {}
+        theta = c.get("rope_theta", together.get("rope_theta", 10000.0))
         scaling = c.get("rope_scaling")
+        if scaling is None and together:
+            scaling = together
         if scaling is not None:
             kind = scaling.get("rope_type", scaling.get("type"))
             if kind in (None, "default"):
@@ -109,7 +116,7 @@ class LlamaConfig:
             num_attention_heads=n_head, num_key_value_heads=n_kv, head_dim=head_dim,
             intermediate_size=inter, vocab_size=int(need("vocab_size")),
             max_position_embeddings=int(c.get("max_position_embeddings", 2048)),
-            rope_theta=float(c.get("rope_theta", 10000.0)),
+            rope_theta=float(theta),
             rms_norm_eps=float(c.get("rms_norm_eps", 1e-5)),
             rope_scaling=scaling,
             tie_word_embeddings=bool(c.get("tie_word_embeddings", False)),

@@ -27,6 +27,15 @@ class Architecture:
     bindings: Callable[[object], list]          # typed configuration -> [weights.Binding]
     config_dict: Callable[[object], dict]       # typed configuration -> config.json dict
     presets: Callable[[str], object] = None     # preset name -> typed configuration
+    # typed configuration -> further CheckpointLayouts under which the same parameters may
+    # be stored (other tensor names); the loader takes the one that fits the files' names
+    other_layouts: Callable[[object], tuple] = None
+
+    def layouts(self, config) -> tuple:
+        """Every layout a checkpoint of ``config`` may have; the first is the one that
+        random weights are written in."""
+        more = tuple(self.other_layouts(config)) if self.other_layouts is not None else ()
+        return (self.bindings(config),) + more
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}

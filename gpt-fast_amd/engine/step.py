@@ -55,7 +55,7 @@ class Engine:
         """Model class by ``config.json``; weights from the folder's safetensors files."""
         arch, config = read_model_folder(folder)
         dev = _device(device)
-        params = load_parameters(folder, arch.bindings(config), dtype, dev)
+        params = load_parameters(folder, arch.layouts(config), dtype, dev)
         return cls.from_plan(arch.plan(config), params, dtype, dev, **cache_args)
 
     @classmethod

@@ -118,8 +118,20 @@ def check_layout(layout: CheckpointLayout, entries: Dict[str, Tuple[str, tuple]]
     return aliased
 
 
-def load_parameters(folder: str, layout: CheckpointLayout, dtype, device) -> Dict[str, torch.Tensor]:
-    """Read every parameter of ``layout`` from the safetensors files of ``folder``."""
+def choose_layout(layouts: Sequence[CheckpointLayout], names) -> CheckpointLayout:
+    """The layout most of whose tensor names are among ``names`` (the first on a tie): a
+    checkpoint is told by the names it uses, and its errors are reported against those."""
+    names = set(names)
+
+    def found(layout):
+        return sum(s.name in names for b in layout.bindings for s in b.sources)
+
+    return max(layouts, key=found)
+
+
+def load_parameters(folder: str, layout, dtype, device) -> Dict[str, torch.Tensor]:
+    """Read every parameter from the safetensors files of ``folder``.  ``layout`` is one
+    :class:`CheckpointLayout` or several, of which the files' tensor names choose."""
     dtype = compute_dtype(dtype)
     files = open_model_files(folder)
     entries, owner = {}, {}
@@ -127,6 +139,8 @@ def load_parameters(folder: str, layout: CheckpointLayout, dtype, device) -> Dic
         for name, meta in f.entries.items():
             entries[name] = meta
             owner[name] = f
+    if not isinstance(layout, CheckpointLayout):
+        layout = choose_layout(tuple(layout), entries)
     aliased = check_layout(layout, entries, folder)
     params: Dict[str, torch.Tensor] = {}
     for b in layout.bindings:

@@ -30,6 +30,14 @@ def test_config_from_keys_and_derivations():
     assert LlamaConfig.from_dict(util.TINY_C).head_dim == 48
     # round trip through config.json keys
     assert LlamaConfig.from_dict(c.to_dict()) == c
+    # the base and the scaling rule kept together under one key read the same
+    moved = {k: v for k, v in util.TINY_B.items() if k not in ("rope_theta", "rope_scaling")}
+    moved["rope_parameters"] = dict(util.TINY_B["rope_scaling"], rope_theta=util.TINY_B["rope_theta"])
+    assert LlamaConfig.from_dict(moved) == c
+    plain_rope = {k: v for k, v in util.TINY_A.items() if k not in ("rope_theta", "rope_scaling")}
+    plain_rope["rope_parameters"] = {"rope_type": "default", "rope_theta": 12345.0}
+    e = LlamaConfig.from_dict(plain_rope)
+    assert e.rope_theta == 12345.0 and e.rope_scaling is None
 
 
 def test_presets_match_reference_registry():          # model.py:44-82
@@ -105,6 +113,43 @@ def test_loader_fuses_and_permutes_like_the_converter(tmp_path):
     assert torch.equal(params["layers.2.feed_forward.w13"][:512], w["layers.2.feed_forward.w1.weight"])
     assert torch.equal(params["layers.2.feed_forward.w13"][512:], w["layers.2.feed_forward.w3.weight"])
     assert params["norm.weight"].dtype == torch.float32
+
+
+def test_loader_takes_the_reference_own_tensor_names(tmp_path):
+    """A checkpoint under the reference's state-dict names (already converted: interleaved
+    rows, fused wqkv; or wq, wk, wv apart, which model.py:184-189 joins as they are) gives
+    the same parameters as the folder it was converted from; the names choose the layout."""
+    folder = _folder(tmp_path, "B")
+    arch, cfg = gfa.read_model_folder(folder)
+    want = load_parameters(folder, arch.layouts(cfg), "float32", None)
+    pcfg, w = plain.load_folder(folder)
+    H, G, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    for split in (False, True):
+        tensors = {}
+        for name, t in w.items():
+            if split and name.endswith("attention.wqkv.weight"):
+                q, k, v = t.split([H * hd, G * hd, G * hd])
+                stem = name[:-len("wqkv.weight")]
+                tensors[stem + "wq.weight"], tensors[stem + "wk.weight"] = q.clone(), k.clone()
+                tensors[stem + "wv.weight"] = v.clone()
+            else:
+                tensors[name] = t.clone()
+        tensors["freqs_cis"] = torch.zeros(4, 2)                        # a buffer: ignored
+        native = str(tmp_path / f"native{int(split)}")
+        os.makedirs(native)
+        write_safetensors(os.path.join(native, "model.safetensors"), tensors)
+        with open(os.path.join(native, "config.json"), "w") as g:
+            json.dump(util.TINY_B, g)
+        got = load_parameters(native, arch.layouts(cfg), "float32", None)
+        assert got.keys() == want.keys()
+        for name in want:
+            assert torch.equal(got[name], want[name]), name
+        # errors are reported in the names the file uses
+        del tensors["layers.1.ffn_norm.weight"]
+        write_safetensors(os.path.join(native, "model.safetensors"), tensors)
+        with pytest.raises(WeightsError) as e:
+            load_parameters(native, arch.layouts(cfg), "float32", None)
+        assert e.value.missing == ["layers.1.ffn_norm.weight"] and not e.value.unexpected
 
 
 def test_loader_dtypes(tmp_path):

@@ -281,10 +281,13 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 
 // --------------------------------------------------------------------------------------
 // Prompts: a workgroup of four waves owns 128 query rows (32 per wave) of one sequence and
-// kv head and walks the keys a page (64 keys) at a time.  The page's keys and values are
-// copied once into LDS by all four waves - each is one contiguous piece of the cache - and
-// the next page is already on its way while the current one is multiplied.  Rows of the
-// LDS tiles are padded so that the operand reads (16 rows at a time) spread over the banks.
+// kv head and walks the keys a page (64 keys) at a time.  A page's keys and values - each
+// one contiguous piece of the cache - are copied by all four waves straight into LDS
+// (global_load_lds, 16 bytes per lane, no registers in between) while earlier pages are
+// multiplied.  An LDS row has no padding; its 16-byte chunks are stored at position
+// (chunk XOR row), chosen on the global side of the copy, so that the operand reads (16
+// rows at a time, the same chunk of each) spread over the banks.
+//
 // The arithmetic is that of the kernel above, a page (64 keys) at a time.
 #define TL_WAVES 4
 #define TL_RT 2
@@ -305,10 +308,12 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         int pair_from) {
     constexpr int DT = DS * 2, RT = TL_RT;
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
-    constexpr int KPITCH = HDM * 2 + 16;                  // bytes per key row in LDS
-    constexpr int VPITCH = 64 * 2 + 16;                   // bytes per value row (one dim, 64 keys)
-    constexpr int KBYTES = 64 * KPITCH, VBYTES = HDM * VPITCH;
-    extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 x (K tile, V tile)
+    constexpr int KROW = HDM * 2;                         // bytes per key row in LDS
+    constexpr int KCH = HDM / 8;                          // 16-byte chunks per key row
+    constexpr int VROW = 64 * 2;                          // bytes per value row (one dim, 64 keys)
+    constexpr int KBYTES = 64 * KROW, VBYTES = HDM * VROW;
+    constexpr int K_PER = KBYTES / 16 / 256, V_PER = VBYTES / 16 / 256;   // copies per thread
+    extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 K tiles, then 2 V tiles
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int seq = blockIdx.z;
@@ -373,74 +378,84 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    // staging: a page's keys are 64 * hd * 2 contiguous bytes, its values hd * 64 * 2
-    const int k_chunks = 64 * hd / 8, v_chunks = hd * 64 / 8;      // 16-byte pieces
-    constexpr int K_PER = (64 * HDM / 8 + 255) / 256, V_PER = (HDM * 64 / 8 + 255) / 256;
-    uint4 kreg[K_PER], vreg[V_PER];
-    int k_dst[K_PER], v_dst[V_PER];                        // LDS byte offsets of this thread's pieces
-    {
-        const int hd8 = hd / 8;                            // 16-byte pieces per key row
+    // Copies.  Thread t fills LDS slots t + 256 i (16 bytes each; a wave's 64 slots are
+    // contiguous, as global_load_lds writes them).  Slot s of a key tile is row s / KCH,
+    // place s % KCH, and holds chunk (place XOR row) of the key that row stands for; keys
+    // are stored in the order the score tiles read them: within a block of 32, key
+    // 8 a + 4 t + b (a < 4, t < 2, b < 4) is row 16 t + 4 a + b, so that the eight scores of
+    // a lane belong to eight consecutive keys (as in the kernel above).  Slot s of a value
+    // tile is dim s / 8, place s % 8, chunk (place XOR dim): keys 8 chunk .. + 7.
+    int k_src[K_PER], v_src[V_PER];                        // byte offsets into the page, -1: nothing
 #pragma unroll
-        for (int i = 0; i < K_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            const int key = c / hd8, piece = c - key * hd8;
-            // keys are stored in the order the score tiles read them: within a block of 32,
-            // key 8 a + 4 t + b (a < 4, t < 2, b < 4) is row 16 t + 4 a + b, so that the
-            // eight scores of a lane belong to eight consecutive keys (as in the kernel above)
-            const int row = (key & 32) | (((key >> 2) & 1) << 4) | (((key >> 3) & 3) << 2) | (key & 3);
-            k_dst[i] = (FULL || c < k_chunks) ? row * KPITCH + piece * 16 : -1;
-        }
-#pragma unroll
-        for (int i = 0; i < V_PER; ++i) {
-            const int c = threadIdx.x + i * 256;
-            v_dst[i] = (FULL || c < v_chunks) ? (c >> 3) * VPITCH + (c & 7) * 16 : -1;   // dim, 8 keys
-        }
+    for (int i = 0; i < K_PER; ++i) {
+        const int slot = threadIdx.x + i * 256;
+        const int row = slot / KCH, chunk = (slot % KCH) ^ (row & (KCH - 1));
+        const int key = (row & 32) | (((row >> 2) & 3) << 3) | (((row >> 4) & 1) << 2) | (row & 3);
+        k_src[i] = (FULL || chunk * 8 < hd) ? (key * hd + chunk * 8) * 2 : -1;
     }
-    auto fetch_page = [&](int pg) {
-        const int page = pages[pg];
-        const uint4* ksrc = (const uint4*)(k_pages + page_row(page, g, 0, Hkv, hd));
-        const uint4* vsrc = (const uint4*)(v_pages + value_elem(page, g, 0, 0, Hkv, hd));
+#pragma unroll
+    for (int i = 0; i < V_PER; ++i) {
+        const int slot = threadIdx.x + i * 256;
+        const int dim = slot >> 3, chunk = (slot & 7) ^ (dim & 7);
+        v_src[i] = (FULL || dim < hd) ? dim * VROW + chunk * 16 : -1;
+    }
+    auto copy_keys = [&](int pg) {
+        const char* src = (const char*)(k_pages + page_row(pages[pg], g, 0, Hkv, hd));
+        char* dst = smem + (pg & 1) * KBYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < K_PER; ++i)
-            kreg[i] = k_dst[i] >= 0 ? ksrc[threadIdx.x + i * 256] : make_uint4(0, 0, 0, 0);
+            if (FULL || k_src[i] >= 0)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(src + k_src[i]),
+                    (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
+    };
+    auto copy_values = [&](int pg) {
+        const char* src = (const char*)(v_pages + value_elem(pages[pg], g, 0, 0, Hkv, hd));
+        char* dst = smem + 2 * KBYTES + (pg & 1) * VBYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < V_PER; ++i)
-            vreg[i] = v_dst[i] >= 0 ? vsrc[threadIdx.x + i * 256] : make_uint4(0, 0, 0, 0);
+            if (FULL || v_src[i] >= 0)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(src + v_src[i]),
+                    (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
     };
-    auto store_page = [&](int buf, int pg) {
-        char* kt = smem + buf * (KBYTES + VBYTES);
-        char* vt = kt + KBYTES;
-        const int keys_ok = wg_pmax - pg * 64;             // keys beyond hold no data yet
-#pragma unroll
-        for (int i = 0; i < K_PER; ++i)
-            if (k_dst[i] >= 0) *(uint4*)(kt + k_dst[i]) = kreg[i];
-        if (keys_ok < 63) {                                // the last page: zero what is not data
-#pragma unroll
-            for (int i = 0; i < V_PER; ++i) {
-                const int piece = (threadIdx.x + i * 256) & 7;
-                Frag f;
-                f.u = vreg[i];
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (piece * 8 + e > keys_ok) f.e[e] = 0;
-                vreg[i] = f.u;
-            }
-        }
+    // The copies of this thread have arrived.  Slots of the newest page that lie beyond the
+    // newest key hold no data yet (whatever the cache held before): their values are set to
+    // zero, by the thread that copied them, so that probability 0 times them is 0.
+    auto copies_landed = [&](int v_pg) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (v_pg > page_hi) return;
+        const int keys_ok = wg_pmax - v_pg * 64;
+        if (keys_ok >= 63) return;
+        char* vt = smem + 2 * KBYTES + (v_pg & 1) * VBYTES;
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
-            if (v_dst[i] >= 0) {
+            const int slot = threadIdx.x + i * 256;
+            const int chunk = (slot & 7) ^ ((slot >> 3) & 7);
+            if ((FULL || v_src[i] >= 0) && chunk * 8 + 7 > keys_ok) {
                 Frag f;
-                f.u = vreg[i];
-                *(uint4*)(vt + v_dst[i]) = f.u;
+                f.u = *(const uint4*)(vt + slot * 16);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (chunk * 8 + e > keys_ok) f.e[e] = 0;
+                *(uint4*)(vt + slot * 16) = f.u;
             }
         }
     };
+
+    // operand reads: this lane's row li of a 16-row tile, chunk c at place c XOR row
+    int k_off[DS], v_off[2];
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) k_off[ds] = li * KROW + (((ds * 4 + lg) ^ (li & (KCH - 1))) << 4);
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) v_off[hb] = li * VROW + (((hb * 4 + lg) ^ (li & 7)) << 4);
+
     // One page (64 keys) at a time: all scores first, then the softmax of both row tiles,
     // then the second product - long enough stretches of independent work for the matrix
     // cores and the vector ALU to overlap inside one wave.
     auto compute_page = [&](int buf, int pg) {
-        const char* kt = smem + buf * (KBYTES + VBYTES);
-        const char* vt = kt + KBYTES;
+        const char* kt = smem + buf * KBYTES;
+        const char* vt = smem + 2 * KBYTES + buf * VBYTES;
         floatx4_t s[RT][4];
 #pragma unroll
         for (int kt16 = 0; kt16 < 4; ++kt16) {
@@ -448,7 +463,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds)
                 kf[ds].u = (FULL || ds * 32 + lg * 8 < hd)
-                               ? *(const uint4*)(kt + (kt16 * 16 + li) * KPITCH + (ds * 32 + lg * 8) * 2)
+                               ? *(const uint4*)(kt + kt16 * 16 * KROW + k_off[ds])
                                : make_uint4(0, 0, 0, 0);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -507,7 +522,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
                 for (int hb = 0; hb < 2; ++hb) {
                     Frag vf;
-                    vf.u = *(const uint4*)(vt + (dt * 16 + li) * VPITCH + (hb * 32 + lg * 8) * 2);
+                    vf.u = *(const uint4*)(vt + dt * 16 * VROW + v_off[hb]);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
                         o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
@@ -516,14 +531,19 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         }
     };
 
-    fetch_page(page_lo);
-    store_page(0, page_lo);
+    // Step pg multiplies page pg while the copies of page pg + 1 are on their way into the
+    // other pair of buffers, which the step before has read last.
+    copy_keys(page_lo);
+    copy_values(page_lo);
+    copies_landed(page_lo);
     __syncthreads();
     for (int pg = page_lo; pg <= page_hi; ++pg) {
-        const int buf = (pg - page_lo) & 1;
-        if (pg < page_hi) fetch_page(pg + 1);
-        if (wave_has_rows && pg * 64 <= pmax && pg * 64 + 63 >= w_lo) compute_page(buf, pg);
-        if (pg < page_hi) store_page(buf ^ 1, pg + 1);
+        if (pg < page_hi) {
+            copy_keys(pg + 1);
+            copy_values(pg + 1);
+        }
+        if (wave_has_rows && pg * 64 <= pmax && pg * 64 + 63 >= w_lo) compute_page(pg & 1, pg);
+        copies_landed(pg + 1);
         __syncthreads();
     }
 
@@ -562,7 +582,7 @@ static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* 
     }
     const int total = (int)(grid.x * grid.y);
     const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
-    const size_t shmem = 2 * (size_t)(64 * (HDM * 2 + 16) + HDM * (64 * 2 + 16));
+    const size_t shmem = 2 * (size_t)(64 * HDM * 2 + HDM * 64 * 2);
     static bool raised = false;
     if (!raised) {
         hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL>,

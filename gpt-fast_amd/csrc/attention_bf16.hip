@@ -457,6 +457,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         const char* kt = smem + buf * KBYTES;
         const char* vt = smem + 2 * KBYTES + buf * VBYTES;
         floatx4_t s[RT][4];
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int kt16 = 0; kt16 < 4; ++kt16) {
             Frag kf[DS];
@@ -473,6 +474,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                     s[rt][kt16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ds].v, qf[rt][ds].v, s[rt][kt16], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         const bool masked = pg * 64 + 63 > pmin || (window > 0 && pg * 64 < pmax - window + 1);
         const int key0 = pg * 64 + lg * 8;                 // this lane's keys: key0 .. +7, key0 + 32 .. +39
         Frag pf[RT][2];
@@ -516,6 +518,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
             }
             l[rt] += sum;
         }
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             if (FULL || dt * 16 < hd) {
@@ -529,6 +532,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                 }
             }
         }
+        __builtin_amdgcn_s_setprio(0);
     };
 
     // Step pg multiplies page pg while the copies of page pg + 1 are on their way into the

@@ -18,7 +18,7 @@ MODULES = ("core", "sampling", "gemm_bf16", "gemm_wide_bf16", "attention_bf16")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-result"]
+         "-Wno-unused-result", "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 class BuildError(RuntimeError):

@@ -615,23 +615,49 @@ extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, cons
 }
 
 // out[row, :] = sum_s w_s o_s / sum_s w_s l_s with w_s = 2^(m_s - max m), splits in order.
-__global__ void attention_combine_kernel(const float* __restrict__ ws_o,
-                                         const float* __restrict__ ws_ml, bf16_t* __restrict__ out,
-                                         int hd, int n_splits, int total_rows) {
-    const int row = blockIdx.x;
-    float mmax = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mmax = fmaxf(mmax, ws_ml[((size_t)s * total_rows + row) * 2]);
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float acc = 0.f, den = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const size_t prow = (size_t)s * total_rows + row;
-            const float ms = ws_ml[prow * 2];
-            if (ms == -INFINITY) continue;            // a split without keys
-            const float wgt = __builtin_amdgcn_exp2f(ms - mmax);
-            den += wgt * ws_ml[prow * 2 + 1];
-            acc += wgt * ws_o[prow * hd + d];
+// One wave per row.  Lane s holds split s's maximum and sum (at most 64 splits); the loads
+// of the partial results do not depend on each other, so a batch of them is in flight at
+// once instead of one round trip per split.
+__global__ __launch_bounds__(64) void attention_combine_kernel(const float* __restrict__ ws_o,
+                                                               const float* __restrict__ ws_ml,
+                                                               bf16_t* __restrict__ out, int hd,
+                                                               int n_splits, int total_rows) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    float ms = -INFINITY, ls = 0.f;
+    if (lane < n_splits) {
+        const float2 ml = *(const float2*)(ws_ml + ((size_t)lane * total_rows + row) * 2);
+        ms = ml.x;
+        ls = ml.y;
+    }
+    const float mmax = wave_max(ms);
+    const float wgt = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);   // a split without keys: 0
+    float den = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) den += __shfl(wgt * ls, sp, 64);
+    const float inv = 1.f / den;
+    for (int d = lane * 2; d < hd; d += 128) {
+        const float* src = ws_o + (size_t)row * hd + d;
+        const size_t stride = (size_t)total_rows * hd;
+        float a0 = 0.f, a1 = 0.f;
+        int sp = 0;
+        for (; sp + 8 <= n_splits; sp += 8) {
+            float2 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = *(const float2*)(src + (sp + j) * stride);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float wj = __shfl(wgt, sp + j, 64);
+                a0 += wj * v[j].x;
+                a1 += wj * v[j].y;
+            }
         }
-        out[(size_t)row * hd + d] = float_to_bf16(acc / den);
+        for (; sp < n_splits; ++sp) {
+            const float2 v = *(const float2*)(src + sp * stride);
+            const float wj = __shfl(wgt, sp, 64);
+            a0 += wj * v.x;
+            a1 += wj * v.y;
+        }
+        out[(size_t)row * hd + d] = float_to_bf16(a0 * inv);
+        out[(size_t)row * hd + d + 1] = float_to_bf16(a1 * inv);
     }
 }
 
@@ -662,7 +688,7 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
                                   int window, int rt, int n_waves, int max_tiles, int n_splits,
                                   hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || max_tiles < 1 ||
+    if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || n_splits > 64 || max_tiles < 1 ||
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
         (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > (rt == 1 ? 8 : 4) ||
         (size_t)(n_waves - 1) * rt * (128 + (hd <= 64 ? 2 : hd <= 128 ? 4 : 8) * 2 * 1024) > 65536)

@@ -8,14 +8,12 @@ from .library import KernelError, check, library, ptr, require_contiguous, requi
 _i = ctypes.c_int
 _f = ctypes.c_float
 
-TARGET_WAVES = 1024        # single-token steps split the context until this many waves run
-MAX_SPLITS = 16
-# A wave takes its keys one 32-key block after another, each a round trip to memory, and the
-# splits are summed by a second kernel whose cost grows with them: up to FEW_SPLITS a wave may
-# be left with 64 keys, beyond that with 128 (measured at contexts of 256 to 4096 keys).
-FEW_SPLITS = 4
-KEYS_PER_WAVE_FEW = 64
-KEYS_PER_WAVE_MANY = 128
+TARGET_WAVES = 2048        # single-token steps split the context until this many waves run
+MAX_SPLITS = 32
+# A wave takes its keys one 32-key block after another, each a round trip to memory; the
+# splits are summed by a second kernel (one wave per row, its loads in flight together), so
+# a wave may be left with as few as 64 keys (measured at contexts of 256 to 16,384 keys).
+KEYS_PER_WAVE = 64
 
 
 TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
@@ -32,9 +30,7 @@ def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int)
         nw = 4 if hd <= 128 else 2
         tiles = (R + 15) // 16
         waves = n_seqs * G * tiles * nw
-        keys = table_width * 64
-        by_keys = max(min(FEW_SPLITS, keys // (KEYS_PER_WAVE_FEW * nw)),
-                      keys // (KEYS_PER_WAVE_MANY * nw))
+        by_keys = table_width * 64 // (KEYS_PER_WAVE * nw)
         splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS, by_keys)
         return rt, nw, tiles, max(splits, 1)
     rt = PREFILL_ROW_TILES if hd <= 128 else min(PREFILL_ROW_TILES, 2)

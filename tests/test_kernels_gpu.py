@@ -257,28 +257,31 @@ def test_attention_finds_one_far_key():
     """One key among hundreds stands out (its score is scaled up): the output must be
     that key's value, wherever in the cache it lies - first row, a page edge, the last."""
     from gpt_fast_amd.ops import attention as A
-    H, G, hd, S = 4, 2, 64, 700
-    for dtype in (torch.float32, torch.bfloat16):
-        for target in (0, 63, 64, 511, 699):
-            k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=target)
-            q = torch.zeros(1, H, hd)
-            for h in range(H):
-                q[0, h] = ks[0][target, h // 2].float() * 40.0
-            q = q.to(dtype)
+    H, G, hd = 4, 2, 64
+    # 700 keys: two context splits in the single-token kernel; 5000 keys: nineteen, summed by
+    # the second kernel in batches of eight and a rest
+    cases = [(dtype, 700, t) for dtype in (torch.float32, torch.bfloat16) for t in (0, 63, 64, 511, 699)]
+    cases += [(torch.bfloat16, 5000, t) for t in (0, 2047, 2600, 4999)]
+    for dtype, S, target in cases:
+        k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=target)
+        q = torch.zeros(1, H, hd)
+        for h in range(H):
+            q[0, h] = ks[0][target, h // 2].float() * 40.0
+        q = q.to(dtype)
 
-            class B:
-                pass
-            batch = B()
-            batch.tok_seq = torch.zeros(1, dtype=torch.int32, device=DEV)
-            batch.tok_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
-            batch.n_tokens = batch.n_seqs = 1
-            batch.max_q_len, batch.max_kv_len, batch.is_decode = 1, S, True
-            batch.q_start = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
-            batch.start_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
-            batch.host_q_start, batch.host_start_pos = [0, 1], [S - 1]
-            out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, 1.0, 0).cpu().float()
-            for h in range(H):
-                close(out[0, h], vs[0][target, h // 2].float(), 2e-2)
+        class B:
+            pass
+        batch = B()
+        batch.tok_seq = torch.zeros(1, dtype=torch.int32, device=DEV)
+        batch.tok_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
+        batch.n_tokens = batch.n_seqs = 1
+        batch.max_q_len, batch.max_kv_len, batch.is_decode = 1, S, True
+        batch.q_start = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+        batch.start_pos = torch.tensor([S - 1], dtype=torch.int32, device=DEV)
+        batch.host_q_start, batch.host_start_pos = [0, 1], [S - 1]
+        out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, 1.0, 0).cpu().float()
+        for h in range(H):
+            close(out[0, h], vs[0][target, h // 2].float(), 2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

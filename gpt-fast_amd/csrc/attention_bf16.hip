@@ -634,8 +634,12 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(const float* __re
     float den = 0.f;
     for (int sp = 0; sp < n_splits; ++sp) den += __shfl(wgt * ls, sp, 64);
     const float inv = 1.f / den;
-    for (int d = lane * 2; d < hd; d += 128) {
-        const float* src = ws_o + (size_t)row * hd + d;
+    // every lane runs the loop (the weights come from other lanes by shuffles); a lane whose
+    // two dims lie beyond the head neither loads nor stores
+    for (int d0 = 0; d0 < hd; d0 += 128) {
+        const int d = d0 + lane * 2;
+        const bool mine = d < hd;
+        const float* src = ws_o + (size_t)row * hd + (mine ? d : 0);
         const size_t stride = (size_t)total_rows * hd;
         float a0 = 0.f, a1 = 0.f;
         int sp = 0;
@@ -656,8 +660,10 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(const float* __re
             a0 += wj * v.x;
             a1 += wj * v.y;
         }
-        out[(size_t)row * hd + d] = float_to_bf16(a0 * inv);
-        out[(size_t)row * hd + d + 1] = float_to_bf16(a1 * inv);
+        if (mine) {
+            out[(size_t)row * hd + d] = float_to_bf16(a0 * inv);
+            out[(size_t)row * hd + d + 1] = float_to_bf16(a1 * inv);
+        }
     }
 }
 

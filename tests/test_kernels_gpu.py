@@ -257,12 +257,14 @@ def test_attention_finds_one_far_key():
     """One key among hundreds stands out (its score is scaled up): the output must be
     that key's value, wherever in the cache it lies - first row, a page edge, the last."""
     from gpt_fast_amd.ops import attention as A
-    H, G, hd = 4, 2, 64
+    H, G = 4, 2
     # 700 keys: two context splits in the single-token kernel; 5000 keys: nineteen, summed by
-    # the second kernel in batches of eight and a rest
-    cases = [(dtype, 700, t) for dtype in (torch.float32, torch.bfloat16) for t in (0, 63, 64, 511, 699)]
-    cases += [(torch.bfloat16, 5000, t) for t in (0, 2047, 2600, 4999)]
-    for dtype, S, target in cases:
+    # the second kernel in batches of eight and a rest; 9000 keys of a small head: thirty-two
+    # splits, more than the lanes that hold the head's dims in that kernel
+    cases = [(dtype, 700, t, 64) for dtype in (torch.float32, torch.bfloat16) for t in (0, 63, 64, 511, 699)]
+    cases += [(torch.bfloat16, 5000, t, 64) for t in (0, 2047, 2600, 4999)]
+    cases += [(torch.bfloat16, 9000, t, 32) for t in (100, 4400, 8999)]
+    for dtype, S, target, hd in cases:
         k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=target)
         q = torch.zeros(1, H, hd)
         for h in range(H):

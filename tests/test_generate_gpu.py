@@ -102,6 +102,33 @@ def test_long_decoding_and_first_tokens(tmp_path_factory):
         assert rel_err(got, want) < tol
 
 
+def test_long_context(tmp_path_factory):
+    """A prompt of 9000 tokens beside a short one, then tokens one by one: 141 pages per
+    sequence, the prompt kernel's last tiles over thousands of keys, and single-token steps
+    whose context is split over 32 workgroups per kv head, float32 and bfloat16."""
+    from gpt_fast_amd import Entry
+    util.TINY["B_long"] = dict(util.TINY_B, max_position_embeddings=16384)
+    S, tail, new = 9000, 50, 24
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        folder = util.make_folder(tmp_path_factory.getbasetemp(), "B_long", seed=3, dtype=dtype)
+        cfg, w = plain.load_folder(folder)
+        tokens = util.random_tokens(cfg["vocab"], S + new, 9)
+        other = util.random_tokens(cfg["vocab"], 300, 10)
+        want = plain.forward(w, cfg, tokens)[S - tail:]
+        eng = engine_for(folder, dtype, max_tokens=64 * 160 * 2)
+        a, b = eng.start_sequence(), eng.start_sequence()
+        got = [eng.step([Entry(b, other[:200]),
+                         Entry(a, tokens[:S], want=list(range(S - tail, S)))]).cpu()]
+        for t in range(new):
+            entries = [Entry(a, [tokens[S + t]], want=[0])]
+            if t < 10:
+                entries.insert(0, Entry(b, [other[200 + t]]))
+            got.append(eng.step(entries).cpu())
+        got = torch.cat(got)
+        assert rel_err(got[:tail], want[:tail]) < tol
+        assert rel_err(got[tail:], want[tail:]) < tol
+
+
 def test_decode_session_with_graph_equals_stepping(tmp_path_factory):
     from gpt_fast_amd import Entry
     from gpt_fast_amd.engine.decode import DecodeSession

@@ -289,9 +289,11 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 // rows at a time, the same chunk of each) spread over the banks.
 //
 // The arithmetic is that of the kernel above, a page (64 keys) at a time.
+// RT row tiles of 16 per wave: 2 (128 rows per workgroup) where the grid exceeds what the chip
+// holds at once and throughput counts (an operand read from LDS then serves two matrix
+// instructions); 1 (64 rows) for grids that are resident at once, where the time is that of
+// the workgroup with the most keys and twice as many, lighter workgroups shorten it.
 #define TL_WAVES 4
-#define TL_RT 2
-#define TL_ROWS (TL_WAVES * TL_RT * 16)
 
 // FULL: the head size is exactly the one the tiles are laid out for (no edge tests).
 // The running maximum of a row is only raised when a block's maximum exceeds it by more than
@@ -299,14 +301,15 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 // bfloat16 operand of the second product hold at full relative precision, and the output
 // accumulators are rescaled rarely instead of nearly every block.
 #define TL_SLACK 8.0f
-template <int DS, bool FULL>
+template <int DS, bool FULL, int RT>
 __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
         bf16_t* __restrict__ out, int H, int Hkv, int hd, float scale_log2, int window,
         int pair_from) {
-    constexpr int DT = DS * 2, RT = TL_RT;
+    constexpr int DT = DS * 2;
+    constexpr int TL_ROWS = TL_WAVES * RT * 16;
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
     constexpr int KROW = HDM * 2;                         // bytes per key row in LDS
     constexpr int KCH = HDM / 8;                          // 16-byte chunks per key row
@@ -571,12 +574,30 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     }
 }
 
-template <int DS, bool FULL>
-static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k,
-                                   const bf16_t* v, const int* q_start, const int* start_pos,
-                                   const int* table, int table_stride, bf16_t* out, int H, int Hkv,
-                                   int hd, float sl2, int window) {
+template <int DS, bool FULL, int RT>
+static void launch_attention_tiled_rt(dim3 grid, int slots, hipStream_t stream, const bf16_t* q,
+                                      const bf16_t* k, const bf16_t* v, const int* q_start,
+                                      const int* start_pos, const int* table, int table_stride,
+                                      bf16_t* out, int H, int Hkv, int hd, float sl2, int window) {
     constexpr int HDM = DS * 32;
+    const int total = (int)(grid.x * grid.y);
+    const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
+    const size_t shmem = 2 * (size_t)(64 * HDM * 2 + HDM * 64 * 2);
+    static bool raised = false;
+    if (!raised) {
+        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL, RT>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        raised = true;
+    }
+    attention_tiled_kernel<DS, FULL, RT><<<grid, 256, shmem, stream>>>(
+        q, k, v, q_start, start_pos, table, table_stride, out, H, Hkv, hd, sl2, window, pair_from);
+}
+
+template <int DS, bool FULL>
+static void launch_attention_tiled(int max_rows, int n_seqs, int row_tiles, hipStream_t stream, const bf16_t* q,
+                                   const bf16_t* k, const bf16_t* v, const int* q_start,
+                                   const int* start_pos, const int* table, int table_stride,
+                                   bf16_t* out, int H, int Hkv, int hd, float sl2, int window) {
     static int slots = 0;                                  // workgroups the chip holds at once
     if (slots == 0) {
         int dev = 0, cus = 0;
@@ -584,33 +605,35 @@ static void launch_attention_tiled(dim3 grid, hipStream_t stream, const bf16_t* 
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         slots = 2 * (cus > 0 ? cus : 1);
     }
-    const int total = (int)(grid.x * grid.y);
-    const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
-    const size_t shmem = 2 * (size_t)(64 * HDM * 2 + HDM * 64 * 2);
-    static bool raised = false;
-    if (!raised) {
-        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        raised = true;
-    }
-    attention_tiled_kernel<DS, FULL><<<grid, 256, shmem, stream>>>(q, k, v, q_start, start_pos, table,
-                                                             table_stride, out, H, Hkv, hd, sl2, window, pair_from);
+    const int tiles128 = (max_rows + 127) / 128;
+    if (row_tiles == 0) row_tiles = ((long)tiles128 * Hkv * n_seqs <= slots) ? 1 : 2;
+    if (row_tiles == 1)                                    // resident at once: lighter workgroups
+        launch_attention_tiled_rt<DS, FULL, 1>(dim3((max_rows + 63) / 64, Hkv, n_seqs), slots, stream, q, k, v,
+                                               q_start, start_pos, table, table_stride, out, H, Hkv, hd, sl2, window);
+    else
+        launch_attention_tiled_rt<DS, FULL, 2>(dim3(tiles128, Hkv, n_seqs), slots, stream, q, k, v, q_start,
+                                               start_pos, table, table_stride, out, H, Hkv, hd, sl2, window);
 }
 
-// Prompts of many rows: max_tiles = most 128-row tiles any sequence needs per kv head.
+// Prompts of many rows: max_rows = most (token, head of a group) rows any sequence has per kv
+// head; row_tiles = 16-row tiles per wave, 1 or 2, or 0 to let the size of the grid choose.
 extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, const void* v_pages,
                                         const int* q_start, const int* start_pos, const int* table,
                                         int table_stride, void* out, int n_tokens, int n_seqs, int H,
-                                        int Hkv, int hd, float scale, int window, int max_tiles,
-                                        hipStream_t stream) {
+                                        int Hkv, int hd, float scale, int window, int max_rows,
+                                        int row_tiles, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_tiles < 1) return (int)hipErrorInvalidValue;
-    const dim3 grid(max_tiles, Hkv, n_seqs);
+    if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_rows < 1 || row_tiles < 0 || row_tiles > 2)
+        return (int)hipErrorInvalidValue;
     const float sl2 = scale * LOG2E;
-    if (hd == 64) launch_attention_tiled<2, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
-    else if (hd < 64) launch_attention_tiled<2, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
-    else if (hd == 128) launch_attention_tiled<4, true>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
-    else launch_attention_tiled<4, false>(grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table, table_stride, (bf16_t*)out, H, Hkv, hd, sl2, window);
+    const bf16_t* qp = (const bf16_t*)q;
+    const bf16_t* kp = (const bf16_t*)k_pages;
+    const bf16_t* vp = (const bf16_t*)v_pages;
+    bf16_t* op = (bf16_t*)out;
+    if (hd == 64) launch_attention_tiled<2, true>(max_rows, n_seqs, row_tiles, stream, qp, kp, vp, q_start, start_pos, table, table_stride, op, H, Hkv, hd, sl2, window);
+    else if (hd < 64) launch_attention_tiled<2, false>(max_rows, n_seqs, row_tiles, stream, qp, kp, vp, q_start, start_pos, table, table_stride, op, H, Hkv, hd, sl2, window);
+    else if (hd == 128) launch_attention_tiled<4, true>(max_rows, n_seqs, row_tiles, stream, qp, kp, vp, q_start, start_pos, table, table_stride, op, H, Hkv, hd, sl2, window);
+    else launch_attention_tiled<4, false>(max_rows, n_seqs, row_tiles, stream, qp, kp, vp, q_start, start_pos, table, table_stride, op, H, Hkv, hd, sl2, window);
     return GFA_LAUNCH_RESULT();
 }
 

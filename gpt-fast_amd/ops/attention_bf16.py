@@ -19,6 +19,7 @@ KEYS_PER_WAVE = 64
 TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
                            # the workgroup-tiled kernel (keys and values through LDS)
 PREFILL_ROW_TILES = 4      # 16-row tiles per wave for prompts
+TILED_ROW_TILES = 0        # of the workgroup-tiled kernel: 1 or 2, or 0 = by the size of the grid
 
 
 def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int):
@@ -61,11 +62,11 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
     R = H // G
     if batch.max_q_len * R >= TILED_MIN_ROWS and hd <= 128:
         out = torch.empty_like(q)
-        tiles = (batch.max_q_len * R + 127) // 128
         check(library("attention_bf16").gfa_attention_tiled_bf16(
             ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos),
             ptr(table), _i(table.shape[1]), ptr(out), _i(n), _i(batch.n_seqs), _i(H), _i(G), _i(hd),
-            _f(scale), _i(window), _i(tiles), stream_handle()), "attention_tiled_bf16")
+            _f(scale), _i(window), _i(batch.max_q_len * R), _i(TILED_ROW_TILES), stream_handle()),
+            "attention_tiled_bf16")
         return out
     rt, nw, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
     out = torch.empty_like(q)

@@ -213,10 +213,19 @@ def _attention_ref(q, k, v, pos, scale, window):
     (7, 7, 32, 0), (10, 2, 112, 0), (9, 3, 96, 65), (5, 1, 144, 0), (2, 2, 176, 0), (3, 1, 208, 0),
     (2, 1, 240, 0), (12, 4, 128, 33), (4, 1, 20, 0), (2, 2, 264, 0),      # last two: plain kernel only
 ])
-def test_attention_over_pages(dtype, tol, H, G, hd, window):
+def test_attention_over_pages(dtype, tol, H, G, hd, window, monkeypatch):
     """Prefill rows (many tokens of a sequence) and decode rows (its last token) in one
-    launch, sequences of unequal length on scattered pages, unused page tails poisoned."""
+    launch, sequences of unequal length on scattered pages, unused page tails poisoned.
+    The workgroup-tiled prompt kernel is run in both its tile heights (a grid this small
+    would only get the lower one)."""
     from gpt_fast_amd.ops import attention as A
+    from gpt_fast_amd.ops import attention_bf16 as AB
+    for row_tiles in ((1, 2) if dtype == torch.bfloat16 else (0,)):
+        monkeypatch.setattr(AB, "TILED_ROW_TILES", row_tiles)
+        _attention_over_pages(A, dtype, tol, H, G, hd, window)
+
+
+def _attention_over_pages(A, dtype, tol, H, G, hd, window):
     lens = [1, 63, 64, 65, 200, 333]
     k_pages, v_pages, table, ks, vs = _paged(lens, G, hd, dtype, seed=hd + H)
     g = torch.Generator().manual_seed(5)
@@ -288,15 +297,18 @@ def test_attention_finds_one_far_key():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n_query", [1, 40])
-def test_attention_window_edge(dtype, n_query):
+def test_attention_window_edge(dtype, n_query, monkeypatch):
     """A window of W keys: the key at distance W - 1 is the last one inside, the key at
     distance W the first one outside.  Two keys are made to stand out, one on each side of
     the edge of the last query: the output must be the inner one's value; with the outer
     one alone in sight of the score, it must not show.  One query row (the decode kernel)
     and forty (the prompt kernel)."""
     from gpt_fast_amd.ops import attention as A
+    from gpt_fast_amd.ops import attention_bf16 as AB
     H, G, hd, S, W = 4, 2, 64, 333, 70
-    for inside in (True, False):
+    both_heights = dtype == torch.bfloat16 and n_query > 1        # of the prompt kernel's tiles
+    for inside, row_tiles in [(i, r) for i in (True, False) for r in ((1, 2) if both_heights else (0,))]:
+        monkeypatch.setattr(AB, "TILED_ROW_TILES", row_tiles)
         k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=17)
         last = S - 1
         edge_in, edge_out = last - W + 1, last - W

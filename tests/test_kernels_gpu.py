@@ -266,18 +266,20 @@ def test_attention_finds_one_far_key():
     """One key among hundreds stands out (its score is scaled up): the output must be
     that key's value, wherever in the cache it lies - first row, a page edge, the last."""
     from gpt_fast_amd.ops import attention as A
-    H, G = 4, 2
     # 700 keys: two context splits in the single-token kernel; 5000 keys: nineteen, summed by
     # the second kernel in batches of eight and a rest; 9000 keys of a small head: thirty-two
-    # splits, more than the lanes that hold the head's dims in that kernel
-    cases = [(dtype, 700, t, 64) for dtype in (torch.float32, torch.bfloat16) for t in (0, 63, 64, 511, 699)]
-    cases += [(torch.bfloat16, 5000, t, 64) for t in (0, 2047, 2600, 4999)]
-    cases += [(torch.bfloat16, 9000, t, 32) for t in (100, 4400, 8999)]
-    for dtype, S, target, hd in cases:
+    # splits, more than the lanes that hold the head's dims in that kernel; then other head
+    # sizes and group sizes (two row tiles per kv head; two waves per workgroup) with splits
+    cases = [(dtype, 700, t, 64, 4, 2) for dtype in (torch.float32, torch.bfloat16) for t in (0, 63, 64, 511, 699)]
+    cases += [(torch.bfloat16, 5000, t, 64, 4, 2) for t in (0, 2047, 2600, 4999)]
+    cases += [(torch.bfloat16, 9000, t, 32, 4, 2) for t in (100, 4400, 8999)]
+    cases += [(torch.bfloat16, 3000, t, hd, H, G) for t in (5, 1500, 2999)
+              for hd, H, G in ((256, 2, 1), (48, 6, 2), (128, 32, 1), (112, 5, 5))]
+    for dtype, S, target, hd, H, G in cases:
         k_pages, v_pages, table, ks, vs = _paged([S], G, hd, dtype, seed=target)
         q = torch.zeros(1, H, hd)
         for h in range(H):
-            q[0, h] = ks[0][target, h // 2].float() * 40.0
+            q[0, h] = ks[0][target, h // (H // G)].float() * 40.0
         q = q.to(dtype)
 
         class B:
@@ -292,7 +294,46 @@ def test_attention_finds_one_far_key():
         batch.host_q_start, batch.host_start_pos = [0, 1], [S - 1]
         out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, 1.0, 0).cpu().float()
         for h in range(H):
-            close(out[0, h], vs[0][target, h // 2].float(), 2e-2)
+            close(out[0, h], vs[0][target, h // (H // G)].float(), 2e-2)
+
+
+@pytest.mark.parametrize("H,G,hd,window", [(8, 2, 128, 0), (4, 4, 64, 0), (6, 2, 96, 0), (8, 2, 128, 1000),
+                                           (3, 1, 48, 0)])
+def test_prompt_attention_over_thousands_of_keys(H, G, hd, window, monkeypatch):
+    """The last 200 tokens of a 3000-token sequence as one prompt step: the workgroup-tiled
+    kernel walks 47 pages per workgroup, in both its tile heights; every 13th row is compared
+    with float64, and the last row must find one far key that stands out."""
+    from gpt_fast_amd.ops import attention as A
+    from gpt_fast_amd.ops import attention_bf16 as AB
+    S, n_q, target = 3000, 200, 2345                      # inside the window of the last row
+    k_pages, v_pages, table, ks, vs = _paged([S], G, hd, torch.bfloat16, seed=hd)
+    g0 = torch.Generator().manual_seed(3)
+    q = torch.randn(n_q, H, hd, generator=g0)
+    for h in range(H):
+        q[-1, h] = ks[0][target, h // (H // G)].float() * (40.0 * math.sqrt(hd))
+    q = bf(q)
+    scale = 1.0 / math.sqrt(hd)
+
+    class B:
+        pass
+    batch = B()
+    pos = list(range(S - n_q, S))
+    batch.tok_seq = torch.zeros(n_q, dtype=torch.int32, device=DEV)
+    batch.tok_pos = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    batch.n_tokens, batch.n_seqs = n_q, 1
+    batch.max_q_len, batch.max_kv_len, batch.is_decode = n_q, S, False
+    batch.q_start = torch.tensor([0, n_q], dtype=torch.int32, device=DEV)
+    batch.start_pos = torch.tensor([S - n_q], dtype=torch.int32, device=DEV)
+    batch.host_q_start, batch.host_start_pos = [0, n_q], [S - n_q]
+    for row_tiles in (1, 2):
+        monkeypatch.setattr(AB, "TILED_ROW_TILES", row_tiles)
+        out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, scale, window).cpu().float()
+        assert not torch.isnan(out).any()
+        for n in list(range(0, n_q - 1, 13)):
+            ref = _attention_ref(q[n].float(), ks[0].float(), vs[0].float(), pos[n], scale, window)
+            close(out[n], ref, 1.5e-2)
+        for h in range(H):
+            close(out[-1, h], vs[0][target, h // (H // G)].float(), 2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

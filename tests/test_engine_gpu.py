@@ -97,3 +97,38 @@ def test_unequal_batches_reuse_slots(tmp_path_factory, name, dtype, tol):
             assert rel_err(torch.cat(got[i]), want) < tol, (name, dtype, round_, i)
         eng.cache.check()
     assert eng.cache.slots.held == 0
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_batch_of_forty_shrinking_to_one(tmp_path_factory, name, dtype, tol):
+    """Forty sequences decode together and end one after another: single-token steps of 40
+    down to 1 rows, which go through the many-row, the few-row and the one-row products."""
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype, max_tokens=64 * 2 * 40)
+    V = util.TINY[name]["vocab_size"]
+    n_seq = 40
+    lengths = [1 + (7 * i) % 23 for i in range(n_seq)]
+    new = [2 + i for i in range(n_seq)]                    # sequence i decodes 2 + i tokens
+    seqs = [util.random_tokens(V, L + n, 300 + i) for i, (L, n) in enumerate(zip(lengths, new))]
+    slots = [eng.start_sequence() for _ in seqs]
+    got = [[] for _ in seqs]
+    logits = eng.step([Entry(s, q[:L], want=[L - 1]) for s, q, L in zip(slots, seqs, lengths)]).cpu()
+    for i in range(n_seq):
+        got[i].append(logits[i:i + 1])
+    live = list(range(n_seq))
+    t = 0
+    while live:
+        logits = eng.step([Entry(slots[i], [seqs[i][lengths[i] + t]], want=[0]) for i in live]).cpu()
+        for row, i in enumerate(live):
+            got[i].append(logits[row:row + 1])
+        t += 1
+        for i in [i for i in live if t >= new[i]]:
+            eng.end_sequence(slots[i])
+            live.remove(i)
+    for i, q in enumerate(seqs):
+        want = util.plain_logits(folder, q)[lengths[i] - 1:]
+        assert rel_err(torch.cat(got[i]), want) < tol, (name, dtype, i)
+    eng.cache.check()
+    assert eng.cache.slots.held == 0

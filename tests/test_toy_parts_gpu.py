@@ -50,14 +50,21 @@ def _steps_equal_whole(eng, toks, want, vocab, tol):
     assert rel_err(torch.cat(got), want) < tol
 
 
-def _plain_attention_block(x, w, prefix, cfg, q_scale=None, k_scale=None, rotate=True):
-    """x + wo(attention(norm(x))) from the plain parts; optional per-position scales on q, k."""
+def _plain_attention_block(x, w, prefix, cfg, q_scale=None, k_scale=None, rotate=True,
+                           kv_of=None):
+    """x + wo(attention(norm(x))) from the plain parts; optional per-position scales on q, k.
+    ``kv_of``: rows whose (normed, projected, rotated) keys and values are used instead of
+    x's own - the input of an earlier run of this layer whose cache is borrowed."""
     S = x.shape[0]
     H, G, hd = cfg["n_head"], cfg["n_kv"], cfg["head_dim"]
     xn = plain.rms_norm(x, w[prefix + "attention_norm.weight"], cfg["eps"])
     qkv = xn @ w[prefix + "attention.wqkv"].T
     q, k, v = qkv.split([H * hd, G * hd, G * hd], dim=-1)
     q, k, v = q.reshape(S, H, hd), k.reshape(S, G, hd), v.reshape(S, G, hd)
+    if kv_of is not None:
+        other = plain.rms_norm(kv_of, w[prefix + "attention_norm.weight"], cfg["eps"])
+        _, k, v = (other @ w[prefix + "attention.wqkv"].T).split([H * hd, G * hd, G * hd], dim=-1)
+        k, v = k.reshape(S, G, hd), v.reshape(S, G, hd)
     if rotate:
         cos, sin = plain.rope_table(torch.arange(S), hd, cfg["rope_base"], cfg["rope_scaling"])
         q, k = plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin)
@@ -213,5 +220,35 @@ def test_toy_position_encoding_that_is_no_rotation():
         else:
             x = _plain_attention_block(x, w, p, pcfg)
         x = _plain_dense_ffn(x, w, p, pcfg)
+    want = plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
+    _steps_equal_whole(eng, toks, want, cfg.vocab_size, TOL_F32)
+
+
+def test_run_order_is_data_a_layer_twice_and_a_borrowed_cache():
+    """order = layer 0, layer 1, layer 1 again (same weights, a cache entry of its own),
+    layer 0 again reading the keys and values its first run wrote (and writing none):
+    compared with the same computation from the plain parts over the whole sequence."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.config.spec import ModelPlan, Run
+    from gpt_fast_amd.parts import Runtime
+    from gpt_fast_amd.parts.model import DecoderModel
+
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_B)
+    base = arch.plan(cfg)
+    plan = ModelPlan(dim=cfg.hidden_size, vocab_size=cfg.vocab_size, layers=list(base.layers[:2]),
+                     order=[Run(0), Run(1), Run(1), Run(0, cache_from=0)], final_norm=base.final_norm)
+    model = DecoderModel(plan, Runtime(torch.float32, DEV))
+    w = _random_parameters(model, 23)
+    eng = gfa.Engine.from_plan(plan, {k: v.to(DEV) for k, v in w.items()}, "float32", DEV,
+                               max_tokens=1024)
+    pcfg = plain.config_from_dict(util.TINY_B)
+    toks = util.random_tokens(cfg.vocab_size, 100, 8)
+    x0 = w["tok_embeddings.weight"][torch.tensor(toks)]
+    x = _plain_dense_ffn(_plain_attention_block(x0, w, "layers.0.", pcfg), w, "layers.0.", pcfg)
+    for _ in range(2):
+        x = _plain_dense_ffn(_plain_attention_block(x, w, "layers.1.", pcfg), w, "layers.1.", pcfg)
+    x = _plain_attention_block(x, w, "layers.0.", pcfg, kv_of=x0)
+    x = _plain_dense_ffn(x, w, "layers.0.", pcfg)
     want = plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
     _steps_equal_whole(eng, toks, want, cfg.vocab_size, TOL_F32)

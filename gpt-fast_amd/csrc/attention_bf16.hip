@@ -280,8 +280,8 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 }
 
 // --------------------------------------------------------------------------------------
-// Prompts: a workgroup of four waves owns 128 query rows (32 per wave) of one sequence and
-// kv head and walks the keys a page (64 keys) at a time.  A page's keys and values - each
+// Prompts: a workgroup of four waves owns 128 or 64 query rows (RT tiles of 16 per wave) of
+// one sequence and kv head and walks the keys a page (64 keys) at a time.  A page's keys and values - each
 // one contiguous piece of the cache - are copied by all four waves straight into LDS
 // (global_load_lds, 16 bytes per lane, no registers in between) while earlier pages are
 // multiplied.  An LDS row has no padding; its 16-byte chunks are stored at position
@@ -453,9 +453,10 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) v_off[hb] = li * VROW + (((hb * 4 + lg) ^ (li & 7)) << 4);
 
-    // One page (64 keys) at a time: all scores first, then the softmax of both row tiles,
-    // then the second product - long enough stretches of independent work for the matrix
-    // cores and the vector ALU to overlap inside one wave.
+    // One page (64 keys) at a time: all scores first, then the softmax of the row tiles, then
+    // the second product.  The wave's priority is raised while it issues matrix instructions,
+    // so that the other waves of the SIMD fill the gaps with their vector work and not the
+    // other way round.
     auto compute_page = [&](int buf, int pg) {
         const char* kt = smem + buf * KBYTES;
         const char* vt = smem + 2 * KBYTES + buf * VBYTES;

@@ -304,11 +304,12 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int j = 0; j < 4; ++j)
                 *(uint4*)(stage + rt * SM_TILE + (lrow + 4 * j) * SM_PITCH + lchunk * 16) = regs[rt][j];
     };
-    // The x fragments of a piece are requested before the prefetch of later pieces of W:
-    // loads return in order, so waiting for x must not mean waiting for the prefetch.
+    // The x fragments of a piece are requested a whole piece ahead, and before the prefetch of
+    // the W piece issued next: loads return in order, so when a piece is multiplied its x has
+    // long been asked for and waiting for it lets two later pieces of W stay in flight.
     constexpr int XS = SM_SUBK / 32;
-    uint4 xraw[XS][CT];                                  // bfloat16 x, or converted below
-    auto load_x = [&](int t) {
+    uint4 x_a[XS][CT], x_b[XS][CT];
+    auto load_x = [&](int t, uint4 (&xraw)[XS][CT]) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             }
         }
     };
-    auto multiply_piece = [&](int t) {
+    auto multiply_piece = [&](int t, const uint4 (&xraw)[XS][CT]) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             Frag8 b[CT];
@@ -338,7 +339,10 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             }
         }
     };
-    if (t_begin < t_end) load_piece(t_begin, regs_a);
+    if (t_begin < t_end) {
+        load_piece(t_begin, regs_a);
+        load_x(t_begin, x_a);
+    }
     if (t_begin + 1 < t_end) load_piece(t_begin + 1, regs_b);
     // What the epilogue of wave 0 reads is requested now, behind the first pieces of W, so
     // that its latency (and the rotation's sine and cosine) passes while W streams.
@@ -396,15 +400,15 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         }
     }
     for (int t = t_begin; t < t_end; t += 2) {
-        load_x(t);
+        if (t + 1 < t_end) load_x(t + 1, x_b);
         stage_piece(regs_a);
         if (t + 2 < t_end) load_piece(t + 2, regs_a);
-        multiply_piece(t);
+        multiply_piece(t, x_a);
         if (t + 1 < t_end) {
-            load_x(t + 1);
+            if (t + 2 < t_end) load_x(t + 2, x_a);
             stage_piece(regs_b);
             if (t + 3 < t_end) load_piece(t + 3, regs_b);
-            multiply_piece(t + 1);
+            multiply_piece(t + 1, x_b);
         }
     }
     if (chained) {                                       // fixed order: lane, lanes of a row, waves

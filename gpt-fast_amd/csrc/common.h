@@ -26,6 +26,14 @@ __device__ __forceinline__ bf16_t float_to_bf16(float f) {
     return __builtin_bit_cast(bf16_t, b);
 }
 
+// 16 bytes of a stream that is read once (the weights): a non-temporal load, so that the
+// lines do not displace x, which every workgroup reads again and again, from the caches.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load16(const void* p) {
+    const u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 template <typename T> __device__ __forceinline__ float load_as_float(const T* p);
 template <> __device__ __forceinline__ float load_as_float<float>(const float* p) { return *p; }
 template <> __device__ __forceinline__ float load_as_float<bf16_t>(const bf16_t* p) {

@@ -105,8 +105,8 @@ __global__ __launch_bounds__(256) void skinny_dot_kernel(
                 Pack8 wa[WR], wb[WR];
 #pragma unroll
                 for (int r = 0; r < WR; ++r) {
-                    wa[r].u = *(const uint4*)(wrow[r] + k0 + c * 8);
-                    wb[r].u = *(const uint4*)(wrow[r] + k0 + (c + 64) * 8);
+                    wa[r].u = stream_load16(wrow[r] + k0 + c * 8);
+                    wb[r].u = stream_load16(wrow[r] + k0 + (c + 64) * 8);
                 }
 #pragma unroll
                 for (int m = 0; m < MT; ++m) {
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void skinny_dot_kernel(
             for (; c < cur8; c += 64) {
                 Pack8 wa[WR];
 #pragma unroll
-                for (int r = 0; r < WR; ++r) wa[r].u = *(const uint4*)(wrow[r] + k0 + c * 8);
+                for (int r = 0; r < WR; ++r) wa[r].u = stream_load16(wrow[r] + k0 + c * 8);
 #pragma unroll
                 for (int m = 0; m < MT; ++m) {
                     Pack8 xa;
@@ -294,8 +294,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                regs[rt][j] = (k < K) ? *(const uint4*)(wsrc[rt][j] + t * SM_SUBK)
-                                      : make_uint4(0, 0, 0, 0);
+                regs[rt][j] = (k < K) ? stream_load16(wsrc[rt][j] + t * SM_SUBK) : make_uint4(0, 0, 0, 0);
     };
     auto stage_piece = [&](uint4 (&regs)[RT][4]) {
 #pragma unroll

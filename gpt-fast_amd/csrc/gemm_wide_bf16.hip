@@ -85,7 +85,7 @@ __global__ __launch_bounds__(NW * 64) void wide_kernel(
         const bool ok = t * WD_SUBK + lchunk * 8 < K;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            regs[j] = ok ? *(const uint4*)(wsrc[j] + (size_t)t * WD_SUBK) : make_uint4(0, 0, 0, 0);
+            regs[j] = ok ? stream_load16(wsrc[j] + (size_t)t * WD_SUBK) : make_uint4(0, 0, 0, 0);
     };
     auto stage_w = [&](uint4 (&regs)[4]) {
 #pragma unroll

@@ -24,9 +24,10 @@ class GatedFeedForward(Part):
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
     prepares_norm = True
-    # x may be an ops.linear.HalfNormed; from two rows on (the one-row gate product runs on
-    # a kernel that takes plain rows and is faster than the saving)
-    takes_prepared = 2
+    # x may be an ops.linear.HalfNormed, from one row on (the least number of rows; with the
+    # weights streamed past the caches the matrix-core kernel that takes the halves is as fast
+    # at one row as the dot-product kernel that does not, and the norm kernel is saved)
+    takes_prepared = 1
 
     def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
         h = L.gated_linear(x, self.w13)

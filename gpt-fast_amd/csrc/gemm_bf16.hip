@@ -254,7 +254,7 @@ struct SkinnyExtra {
 // Rows per record of the sums-of-squares shares for M rows of x.
 extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-template <int CT, int MODE>
+template <int CT, int MODE, int XP = 1>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, SkinnyExtra ex) {
@@ -306,28 +306,52 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     // The x fragments of a piece are requested a whole piece ahead, and before the prefetch of
     // the W piece issued next: loads return in order, so when a piece is multiplied its x has
     // long been asked for and waiting for it lets two later pieces of W stay in flight.
+    //
+    // XP = 2 or 4 (at most eight or four rows of x, CT == 1): the other columns of the x
+    // operand stand for no row, and what a matrix instruction makes of them is never stored.
+    // So the sixteen lanes of a group are 16 / XP rows times XP steps of 32 k: part q of the
+    // lanes loads, in the same instruction, the chunk that part 0 needs q steps later - the
+    // next pieces of the rows' 128-byte lines - and a rotation of the group by q * 16 / XP
+    // lanes brings it down when that step is multiplied: 1 / XP of the load instructions
+    // for x, each using whole lines.
     constexpr int XS = SM_SUBK / 32;
-    uint4 x_a[XS][CT], x_b[XS][CT];
-    auto load_x = [&](int t, uint4 (&xraw)[XS][CT]) {
+    constexpr int XL = XS / XP;                          // loads of x per piece and tile of rows
+    constexpr int XROWS = 16 / XP;
+    static_assert(XP == 1 || CT == 1, "shared operand columns need a single tile of rows");
+    uint4 x_a[XL][CT], x_b[XL][CT];
+    auto load_x = [&](int t, uint4 (&xraw)[XL][CT]) {
 #pragma unroll
-        for (int s = 0; s < XS; ++s) {
-            const int kk = t * SM_SUBK + (s * 4 + fg) * 8;
-            {
+        for (int s = 0; s < XL; ++s) {
+            const int kk = t * SM_SUBK + ((XP * s + fi / XROWS) * 4 + fg) * 8;
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    const int m = ct * 16 + fi;
-                    xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
-                                                    : make_uint4(0, 0, 0, 0);
-                }
+            for (int ct = 0; ct < CT; ++ct) {
+                const int m = ct * 16 + fi % XROWS;
+                xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
+                                                : make_uint4(0, 0, 0, 0);
             }
         }
     };
-    auto multiply_piece = [&](int t, const uint4 (&xraw)[XS][CT]) {
+    // lanes i of every group of sixteen get the value of lane (i + N) mod 16
+    #define GFA_ROTATE_DOWN(v, N) __builtin_amdgcn_update_dpp(0, (int)(v), 0x120 + ((16 - (N)) & 15), 0xf, 0xf, false)
+    auto multiply_piece = [&](int t, const uint4 (&xraw)[XL][CT]) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             Frag8 b[CT];
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s][ct];
+            for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s / XP][ct];
+            if (XP > 1 && s % XP != 0) {
+                const int q = s % XP;
+                if (q * XROWS == 4) {
+                    b[0].u.x = GFA_ROTATE_DOWN(b[0].u.x, 4); b[0].u.y = GFA_ROTATE_DOWN(b[0].u.y, 4);
+                    b[0].u.z = GFA_ROTATE_DOWN(b[0].u.z, 4); b[0].u.w = GFA_ROTATE_DOWN(b[0].u.w, 4);
+                } else if (q * XROWS == 8) {
+                    b[0].u.x = GFA_ROTATE_DOWN(b[0].u.x, 8); b[0].u.y = GFA_ROTATE_DOWN(b[0].u.y, 8);
+                    b[0].u.z = GFA_ROTATE_DOWN(b[0].u.z, 8); b[0].u.w = GFA_ROTATE_DOWN(b[0].u.w, 8);
+                } else {
+                    b[0].u.x = GFA_ROTATE_DOWN(b[0].u.x, 12); b[0].u.y = GFA_ROTATE_DOWN(b[0].u.y, 12);
+                    b[0].u.z = GFA_ROTATE_DOWN(b[0].u.z, 12); b[0].u.w = GFA_ROTATE_DOWN(b[0].u.w, 12);
+                }
+            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 Frag8 a;
@@ -338,6 +362,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             }
         }
     };
+    #undef GFA_ROTATE_DOWN
     if (t_begin < t_end) {
         load_piece(t_begin, regs_a);
         load_x(t_begin, x_a);
@@ -561,21 +586,25 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         exl.share_off = (int)shmem;
         shmem += (size_t)nw * 16 * 64 * sizeof(float);
     }
-#define GFA_LAUNCH_MFMA(CTV)                                                                      \
+#define GFA_LAUNCH_MFMA(CTV, XPV)                                                                 \
     do {                                                                                          \
         static bool raised = false;                                                               \
         if (!raised) {                                                                            \
-            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE>,                 \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV>,                  \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
+        skinny_mfma_kernel<CTV, MODE, XPV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
     } while (0)
     switch (ct) {
-        case 1: GFA_LAUNCH_MFMA(1); break;
-        case 2: GFA_LAUNCH_MFMA(2); break;
-        case 3: GFA_LAUNCH_MFMA(3); break;
-        default: GFA_LAUNCH_MFMA(4); break;
+        case 1:                                          // columns of the x operand that stand
+            if (M <= 4) GFA_LAUNCH_MFMA(1, 4);             // for no row carry later steps of k
+            else if (M <= 8) GFA_LAUNCH_MFMA(1, 2);
+            else GFA_LAUNCH_MFMA(1, 1);
+            break;
+        case 2: GFA_LAUNCH_MFMA(2, 1); break;
+        case 3: GFA_LAUNCH_MFMA(3, 1); break;
+        default: GFA_LAUNCH_MFMA(4, 1); break;
     }
 #undef GFA_LAUNCH_MFMA
     return GFA_LAUNCH_RESULT();

@@ -87,7 +87,7 @@ def test_gemm_f32(M, N, K_):
     close(res, keep.double() + ref, 1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K_", [(40, 64), (136, 200), (1000, 328), (96, 4096), (77, 75)])
 def test_skinny_bf16(M, N, K_):
     from gpt_fast_amd.ops import gemm_bf16 as G

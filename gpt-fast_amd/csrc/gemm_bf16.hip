@@ -5,8 +5,10 @@
 // organised around that stream: every wavefront owns a few rows of W and reads them
 // front to back in 16-byte pieces per lane (1 KiB contiguous per wave and load), keeps
 // one float accumulator per (row of W, row of x) and reduces over the lanes at the end.
-// x is small and stays in cache.  Products use v_dot2_f32_bf16 (two multiply-adds per
-// lane and instruction, float accumulate).
+// x is small and stays in cache: W is read with non-temporal loads so that the stream does
+// not displace it, for every workgroup reads all of x again.  One row uses v_dot2_f32_bf16
+// (two multiply-adds per lane and instruction, float accumulate); more rows the matrix cores
+// (second kernel below).
 //
 // Epilogues (MODE): 0 store bfloat16, 1 store float, 2 add into a float matrix (the
 // residual stream), 3 gate: out[m, n] = silu(x W[n]) * (x W[n + gate_rows]) in bfloat16

@@ -256,7 +256,7 @@ struct SkinnyExtra {
 // Rows per record of the sums-of-squares shares for M rows of x.
 extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-template <int CT, int MODE, int XP = 1>
+template <int CT, int MODE, int XP = 1, bool XF = false>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, SkinnyExtra ex) {
@@ -324,23 +324,45 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     auto load_x = [&](int t, uint4 (&xraw)[XL][CT]) {
 #pragma unroll
         for (int s = 0; s < XL; ++s) {
-            const int kk = t * SM_SUBK + ((XP * s + fi / XROWS) * 4 + fg) * 8;
+            // XF: load s of a pair takes rows 8 (s & 1) .. + 7, its lanes 8..15 the later step
+            const int kk = XF ? t * SM_SUBK + (((s & ~1) + (fi >> 3)) * 4 + fg) * 8
+                              : t * SM_SUBK + ((XP * s + fi / XROWS) * 4 + fg) * 8;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const int m = ct * 16 + fi % XROWS;
+                const int m = XF ? ct * 16 + 8 * (s & 1) + (fi & 7) : ct * 16 + fi % XROWS;
                 xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
                                                 : make_uint4(0, 0, 0, 0);
             }
         }
     };
+    // XF (nine to sixteen rows, XP == 1): every column of the operand is a row, but a load can
+    // still use whole lines: of a pair of steps, the first load takes rows 0..7 and the second
+    // rows 8..15, in each the lanes 8..15 the later step; halves are exchanged by the same
+    // rotation when a step is multiplied.
     // lanes i of every group of sixteen get the value of lane (i + N) mod 16
     #define GFA_ROTATE_DOWN(v, N) __builtin_amdgcn_update_dpp(0, (int)(v), 0x120 + ((16 - (N)) & 15), 0xf, 0xf, false)
     auto multiply_piece = [&](int t, const uint4 (&xraw)[XL][CT]) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
             Frag8 b[CT];
+            if (XF) {
+                // rows 0..7 of step s sit in the pair's first load (lanes 0..7 if s is even,
+                // 8..15 if odd), rows 8..15 in its second: own lanes or the other half's
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s / XP][ct];
+                for (int ct = 0; ct < CT; ++ct) {
+                    const uint4 lo = xraw[s & ~1][ct], hi = xraw[s | 1][ct];
+                    const uint4 moved = (s & 1) ? lo : hi;     // the one that has to change halves
+                    uint4 r;
+                    r.x = GFA_ROTATE_DOWN(moved.x, 8); r.y = GFA_ROTATE_DOWN(moved.y, 8);
+                    r.z = GFA_ROTATE_DOWN(moved.z, 8); r.w = GFA_ROTATE_DOWN(moved.w, 8);
+                    const bool low = fi < 8;
+                    const uint4 a0 = (s & 1) ? r : lo, a1 = (s & 1) ? hi : r;
+                    b[ct].u = make_uint4(low ? a0.x : a1.x, low ? a0.y : a1.y, low ? a0.z : a1.z, low ? a0.w : a1.w);
+                }
+            } else {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s / XP][ct];
+            }
             if (XP > 1 && s % XP != 0) {
                 const int q = s % XP;
                 if (q * XROWS == 4) {
@@ -588,25 +610,25 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         exl.share_off = (int)shmem;
         shmem += (size_t)nw * 16 * 64 * sizeof(float);
     }
-#define GFA_LAUNCH_MFMA(CTV, XPV)                                                                 \
+#define GFA_LAUNCH_MFMA(CTV, XPV, XFV)                                                                 \
     do {                                                                                          \
         static bool raised = false;                                                               \
         if (!raised) {                                                                            \
-            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV>,                  \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV, XFV>,                  \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, XPV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
+        skinny_mfma_kernel<CTV, MODE, XPV, XFV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
     } while (0)
     switch (ct) {
         case 1:                                          // columns of the x operand that stand
-            if (M <= 4) GFA_LAUNCH_MFMA(1, 4);             // for no row carry later steps of k
-            else if (M <= 8) GFA_LAUNCH_MFMA(1, 2);
-            else GFA_LAUNCH_MFMA(1, 1);
+            if (M <= 4) GFA_LAUNCH_MFMA(1, 4, false);      // for no row carry later steps of k
+            else if (M <= 8) GFA_LAUNCH_MFMA(1, 2, false);
+            else GFA_LAUNCH_MFMA(1, 1, true);
             break;
-        case 2: GFA_LAUNCH_MFMA(2, 1); break;
-        case 3: GFA_LAUNCH_MFMA(3, 1); break;
-        default: GFA_LAUNCH_MFMA(4, 1); break;
+        case 2: GFA_LAUNCH_MFMA(2, 1, false); break;
+        case 3: GFA_LAUNCH_MFMA(3, 1, false); break;
+        default: GFA_LAUNCH_MFMA(4, 1, false); break;
     }
 #undef GFA_LAUNCH_MFMA
     return GFA_LAUNCH_RESULT();

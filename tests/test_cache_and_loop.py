@@ -299,3 +299,24 @@ def test_bench_refuses_more_than_one_gpu_in_one_line():
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 2
     assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
+
+
+def test_attention_plan_for_single_token_steps():
+    """How a single-token step is cut over waves: pure arithmetic, no kernel.  More sequences
+    mean fewer context splits; a split never leaves a wave less than 64 keys of the table's
+    capacity, never exceeds 32, and short contexts are not split at all."""
+    from gpt_fast_amd.ops.attention_bf16 import MAX_SPLITS, plan
+    H, G, hd = 32, 8, 128
+    for n_seqs in (1, 3, 8, 64, 300):
+        for width in (1, 4, 17, 65, 257, 2048):
+            rt, nw, tiles, splits = plan(n_seqs, 1, H, G, hd, width)
+            assert rt == 1 and tiles == 1 and nw == 4
+            assert 1 <= splits <= MAX_SPLITS
+            assert splits == 1 or splits * nw * 64 <= width * 64
+    assert plan(1, 1, H, G, hd, 4)[3] == 1
+    assert plan(1, 1, H, G, hd, 65)[3] == 16 and plan(1, 1, H, G, hd, 257)[3] == 32
+    assert plan(64, 1, H, G, hd, 65)[3] == 1
+    assert plan(8, 1, H, G, hd, 65)[3] == 8
+    # 32 query heads on one kv head: two row tiles per token; wide heads: two waves
+    assert plan(2, 1, 32, 1, 64, 8)[2] == 2
+    assert plan(2, 1, 4, 2, 256, 8)[1] == 2

@@ -8,8 +8,8 @@ generated tokens, through hand-written HIP kernels for gfx950:
     out = generate(engine, [[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
 """
 from . import architectures as _architectures          # registers the known architectures
-from .config.registry import (architecture, known_architectures, read_model_folder,
-                              register_architecture)
+from .config.registry import (architecture, find_preset, known_architectures,
+                              read_model_folder, register_architecture)
 from .engine.batch import Entry
 from .engine.step import Engine
 from .parts.base import (register_block, register_feed_forward, register_mixer, register_norm,

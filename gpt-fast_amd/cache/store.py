@@ -17,7 +17,8 @@ Runs with equal needs form a *group* with storage of its own:
   key in them is out of reach.  Pages are reused without clearing: a reader never looks
   beyond a sequence's length (the reference relies on the same masking when it reuses its
   buffers, model.py:118-119).
-* a state group owns ``[entries, n_slots, *shape]``.
+* a state group owns ``[entries, n_slots + 1, *shape]``; the last slot belongs to no
+  sequence (rows that only fill a recorded batch's shape use it).
 
 The reference's cache is one ``[batch, heads, max_len, head_dim]`` buffer pair per layer
 with one shared position for all rows (model.py:84-100, 117-134); here every sequence has
@@ -76,7 +77,9 @@ class StateGroup:
     def __init__(self, need: StateNeed, entries: int, n_slots: int, device):
         self.need = need
         self.entries = entries
-        self.data = torch.zeros((entries, n_slots) + tuple(need.shape),
+        # one slot beyond the pool (index n_slots) belongs to no sequence: rows of a batch
+        # that only fill a fixed shape read and write it
+        self.data = torch.zeros((entries, n_slots + 1) + tuple(need.shape),
                                 dtype=getattr(torch, need.dtype), device=device)
 
 
@@ -99,7 +102,7 @@ class CacheEntry:
 
     @property
     def state(self) -> torch.Tensor:
-        """[n_slots, *shape] of a state group."""
+        """[n_slots + 1, *shape] of a state group; the last row is the spare slot."""
         return self.group.data[self.index]
 
 
@@ -121,6 +124,7 @@ class Cache:
         self.dtype = dtype
         self.device = device
         self.slots = FreeList(max_sequences, "sequence slot")
+        self.spare_slot = max_sequences         # of state groups; belongs to no sequence
         self.lengths: List[int] = [0] * max_sequences
 
         order_of_need: Dict[object, int] = {}
@@ -234,6 +238,22 @@ class Cache:
 
     def page_list(self, group_id: int, slot: int) -> List[int]:
         return self.groups[group_id].held[slot]
+
+    @property
+    def state_groups(self) -> List[Tuple[int, StateGroup]]:
+        return [(i, g) for i, g in enumerate(self.groups) if isinstance(g, StateGroup)]
+
+    def require_room(self, lengths: Sequence[int]) -> None:
+        """Raise :class:`CacheFull` unless sequences that grow to these lengths fit together
+        in an empty cache (slots and, for every group, pages)."""
+        if len(lengths) > self.max_sequences:
+            raise CacheFull(f"{len(lengths)} sequences at once, but the cache has "
+                            f"{self.max_sequences} slots")
+        need = sum(pages_for(n) for n in lengths)
+        if need > self.n_pages:
+            raise CacheFull(
+                f"the cache holds {self.n_pages * PAGE} tokens in pages of {PAGE}; sequences "
+                f"of {list(lengths)} tokens need {need * PAGE}")
 
     def tokens_held(self) -> int:
         """Tokens of all live sequences, each rounded up to whole pages."""

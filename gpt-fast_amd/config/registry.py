@@ -59,6 +59,32 @@ def architecture(name: str) -> Architecture:
             f"unknown architecture '{name}'; known: {known_architectures()}") from None
 
 
+def find_preset(name: str, architecture_name: str = None):
+    """(architecture, typed configuration) of a named preset.  With ``architecture_name``
+    that architecture's presets are asked; else every registered architecture's, and the
+    name must be known to exactly one of them."""
+    if architecture_name is not None:
+        arch = architecture(architecture_name)
+        if arch.presets is None:
+            raise UnknownArchitecture(f"architecture '{architecture_name}' has no presets")
+        return arch, arch.presets(name)
+    found, errors = [], []
+    for arch in {id(a): a for a in _ARCHITECTURES.values()}.values():
+        if arch.presets is None:
+            continue
+        try:
+            found.append((arch, arch.presets(name)))
+        except (KeyError, ValueError) as e:
+            errors.append(str(e))
+    if not found:
+        raise UnknownArchitecture(f"no architecture has a preset '{name}': " + "; ".join(errors))
+    if len(found) > 1:
+        raise UnknownArchitecture(
+            f"preset '{name}' is known to several architectures "
+            f"({', '.join(a.names[0] for a, _ in found)}); name one")
+    return found[0]
+
+
 def architecture_of(config_json: dict) -> Architecture:
     """The architecture that a ``config.json`` dictionary names."""
     names = list(config_json.get("architectures") or [])

@@ -9,8 +9,8 @@ architecture's name.  Every size and constant a part needs is a field of its spe
 A spec's ``kind`` selects the part class in the registries of ``parts``; a test or an
 application can define a new spec class with a new ``kind`` and register a part for it.
 """
-from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Tuple
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -96,7 +96,8 @@ class Run:
 
 @dataclass
 class ModelPlan:
-    """A whole decoder: embedding, layers in run order, final norm, output head."""
+    """A whole decoder: embedding, layers in run order, final norm, output head.
+    ``max_positions`` bounds prompt + new tokens of a generated request."""
     dim: int
     vocab_size: int
     layers: List[LayerSpec]
@@ -108,7 +109,13 @@ class ModelPlan:
     final_norm_name: str = "norm.weight"
     head_name: str = "output.weight"
     stop_tokens: Tuple[int, ...] = ()
-    extra: Dict[str, object] = field(default_factory=dict)
+    # Optional steps around the layers; None leaves the step out (the reference has none
+    # of them, model.py:136-146).
+    embedding_scale: Optional[float] = None     # embedded rows are multiplied by this
+    input_position: object = None               # a position spec whose part adds to the embedded
+    input_position_name: str = "input_position"  # rows (``add_to_stream``); prefix of its tensors
+    logit_scale: Optional[float] = None         # logits are multiplied by this,
+    logit_softcap: Optional[float] = None       # then capped: cap * tanh(logits / cap)
 
     def validate(self) -> None:
         if not self.layers:

@@ -1,10 +1,13 @@
 """Compiling the HIP sources of this folder for gfx950 into shared libraries.
 
 Each ``<name>.hip`` becomes ``build/libgfa_<name>.so`` (plain ``hipcc -shared``, C entry
-points, no Python headers).  ``ensure(names)`` compiles only the libraries that are
-asked for and not yet built; ``build_all()`` compiles every one anew.  Nothing here
-needs a GPU: hipcc cross-compiles.
+points, no Python headers) with a stamp file beside it that holds a hash of what it was
+built from (the source, ``common.h``, the flags).  ``ensure(names)`` compiles the libraries
+that are asked for and are missing or whose stamp no longer fits the sources, so an edited
+kernel is never run from an old library; ``build_all()`` compiles every one anew.  Nothing
+here needs a GPU: hipcc cross-compiles.
 """
+import hashlib
 import os
 import shutil
 import subprocess
@@ -46,11 +49,38 @@ def _build_dir() -> str:
         return d
 
 
+def source_hash(name: str) -> str:
+    """Hash of everything the library of module ``name`` is built from."""
+    h = hashlib.sha256()
+    for path in (os.path.join(HERE, name + ".hip"), os.path.join(HERE, "common.h")):
+        with open(path, "rb") as f:
+            h.update(f.read())
+        h.update(b"\0")
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()
+
+
+def _is_current(path: str, name: str) -> bool:
+    """The library at ``path`` exists and was built from the sources as they are now."""
+    if not os.path.isfile(path):
+        return False
+    try:
+        with open(path + ".stamp") as f:
+            return f.read().strip() == source_hash(name)
+    except OSError:
+        return False
+
+
+def _candidates(name: str):
+    yield os.path.join(HERE, "build", f"libgfa_{name}.so")
+    yield os.path.join(tempfile.gettempdir(), f"gfa_build_{os.getuid()}", f"libgfa_{name}.so")
+
+
 def library_path(name: str) -> str:
-    """Where the built library of module ``name`` is, or would be put."""
-    in_tree = os.path.join(HERE, "build", f"libgfa_{name}.so")
-    if os.path.isfile(in_tree):
-        return in_tree
+    """Where the current library of module ``name`` is, or would be put."""
+    for path in _candidates(name):
+        if _is_current(path, name):
+            return path
     return os.path.join(_build_dir(), f"libgfa_{name}.so")
 
 
@@ -63,6 +93,7 @@ def _hipcc() -> str:
 
 def _compile(name: str, out: str, log) -> None:
     src = os.path.join(HERE, name + ".hip")
+    stamp = source_hash(name)                         # of the sources as they are compiled
     tmp = out + f".tmp{os.getpid()}"
     cmd = [_hipcc()] + FLAGS + ["-I", HERE, src, "-o", tmp]
     env = dict(os.environ)
@@ -84,6 +115,9 @@ def _compile(name: str, out: str, log) -> None:
             os.remove(tmp)
         raise BuildError(f"hipcc failed on {name}.hip:\n{output}")
     os.replace(tmp, out)
+    with open(out + ".stamp.tmp", "w") as f:
+        f.write(stamp)
+    os.replace(out + ".stamp.tmp", out + ".stamp")
 
 
 def build(names, force=False, log=None) -> None:
@@ -92,11 +126,8 @@ def build(names, force=False, log=None) -> None:
     for n in names:
         if n not in available_modules():
             raise BuildError(f"no source {n}.hip in {HERE}")
-        path = library_path(n)
-        if force or not os.path.isfile(path):
-            if force:
-                path = os.path.join(_build_dir(), f"libgfa_{n}.so")
-            todo.append((n, path))
+        if force or not _is_current(library_path(n), n):
+            todo.append((n, os.path.join(_build_dir(), f"libgfa_{n}.so")))
     if not todo:
         return
     log(f"[gpt_fast_amd] compiling {', '.join(n for n, _ in todo)} for {ARCH} ...")
@@ -119,7 +150,7 @@ def build(names, force=False, log=None) -> None:
 
 
 def ensure(names) -> None:
-    """Build the named libraries if they are not there yet."""
+    """Build the named libraries that are missing or older than their sources."""
     build(names, force=False)
 
 

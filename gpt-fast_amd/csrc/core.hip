@@ -596,6 +596,25 @@ extern "C" int gfa_add_into(float* res, const void* y, size_t total, int y_bf16,
 }
 
 // --------------------------------------------------------------------------------------
+// x[e] = scale * x[e], then, if cap > 0, cap * tanh(x[e] / cap): a factor on the embedded
+// rows or on the logits, and a soft cap of the logits, for plans that state one.
+__global__ void scale_cap_kernel(float* __restrict__ x, size_t total, float scale, float cap) {
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
+         e += (size_t)gridDim.x * blockDim.x) {
+        float v = x[e] * scale;
+        if (cap > 0.f) v = cap * tanhf(v / cap);
+        x[e] = v;
+    }
+}
+
+extern "C" int gfa_scale_cap(float* x, size_t total, float scale, float cap, hipStream_t stream) {
+    if (total == 0) return 0;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    scale_cap_kernel<<<blocks, 256, 0, stream>>>(x, total, scale, cap);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
 // naive matrix product with bfloat16 operands and float accumulation, one thread per
 // output: the plain counterpart of the fast bfloat16 kernels (tests only).
 __global__ void gemm_bf16_naive_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,

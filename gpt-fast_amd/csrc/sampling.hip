@@ -91,14 +91,18 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
         const float* __restrict__ logits, size_t row_stride, int V, float temperature, int top_k,
-        uint32_t seed_lo, uint32_t seed_hi, const int* __restrict__ row_keys,
-        const int* __restrict__ positions, int position_offset, int* __restrict__ out,
-        float* __restrict__ probs_out) {
+        uint32_t seed_lo, uint32_t seed_hi, const uint32_t* __restrict__ seed_dev,
+        const int* __restrict__ row_keys, const int* __restrict__ positions, int position_offset,
+        int* __restrict__ out, float* __restrict__ probs_out) {
     __shared__ ArgBest scratch[16];
     __shared__ float fscratch[16];
     __shared__ unsigned hist[256];
     __shared__ uint32_t sh_prefix;
     __shared__ int sh_remaining;
+    if (seed_dev) {                  // the seed lives in device memory: a recorded launch
+        seed_lo = seed_dev[0];       // can be replayed with another seed
+        seed_hi = seed_dev[1];
+    }
     const int b = blockIdx.x;
     const float* row = logits + b * row_stride;
     const float t = fmaxf(temperature, 1e-5f);
@@ -176,14 +180,15 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     if (threadIdx.x == 0) out[b] = best.i < 0 ? 0 : best.i;
 }
 
+// `seed_dev`: null, or two 32-bit words in device memory (low, high) that replace `seed`.
 extern "C" int gfa_sample(const float* logits, size_t row_stride, int n_rows, int V,
-                          float temperature, int top_k, uint64_t seed, const int* row_keys,
-                          const int* positions, int position_offset, int* out, float* probs_out,
-                          hipStream_t stream) {
+                          float temperature, int top_k, uint64_t seed, const uint32_t* seed_dev,
+                          const int* row_keys, const int* positions, int position_offset, int* out,
+                          float* probs_out, hipStream_t stream) {
     if (n_rows <= 0) return 0;
     sample_kernel<<<n_rows, SMP_THREADS, 0, stream>>>(
         logits, row_stride, V, temperature, top_k, (uint32_t)(seed & 0xffffffffu),
-        (uint32_t)(seed >> 32), row_keys, positions, position_offset, out, probs_out);
+        (uint32_t)(seed >> 32), seed_dev, row_keys, positions, position_offset, out, probs_out);
     return GFA_LAUNCH_RESULT();
 }
 
@@ -192,7 +197,9 @@ extern "C" int gfa_sample(const float* logits, size_t row_stride, int n_rows, in
 // workgroup per chunk of SPL_CHUNK logits, a handful of small launches whose partial
 // results meet in a workspace.  Integer histograms are summed with atomics (the sum does
 // not depend on the order); float partials are added in chunk order.  Workspace, per row:
-//   int   hist[4][256]   (zeroed by the caller)      int   state[2] = {prefix key, remaining}
+//   int   hist[4][256]   (zero before the call; the kernel that reads a histogram clears it,
+//                         so a workspace that was zero once stays usable call after call)
+//   int   state[2] = {prefix key, remaining}
 //   float pmax[NB], psum[NB], pbest_v[NB]            int   pbest_i[NB]
 #define SPL_CHUNK 4096
 #define SPL_THREADS 1024
@@ -264,6 +271,7 @@ __global__ __launch_bounds__(256) void split_pick_kernel(int pass, int top_k, Sp
     }
     const unsigned rem = pass == 0 ? (unsigned)top_k : ws.state[b * 2 + 1];
     const unsigned prefix = pass == 0 ? 0u : ws.state[b * 2];
+    ws.hist[(b * 4 + pass) * 256 + t] = 0;             // read above; zero again for the next call
     __syncthreads();
     if (suffix[t] >= rem && suffix[t + 1] < rem) {     // exactly one bin
         ws.state[b * 2] = prefix | ((unsigned)t << (24 - 8 * pass));
@@ -299,11 +307,15 @@ __global__ __launch_bounds__(SPL_THREADS) void split_sum_kernel(
 // probabilities, the exponential race, and each chunk's best candidate
 __global__ __launch_bounds__(SPL_THREADS) void split_race_kernel(
         const float* __restrict__ logits, size_t row_stride, int V, float t, int use_pivot,
-        uint32_t seed_lo, uint32_t seed_hi, const int* __restrict__ row_keys,
-        const int* __restrict__ positions, int position_offset, float* __restrict__ probs_out,
-        SplitWs ws) {
+        uint32_t seed_lo, uint32_t seed_hi, const uint32_t* __restrict__ seed_dev,
+        const int* __restrict__ row_keys, const int* __restrict__ positions, int position_offset,
+        float* __restrict__ probs_out, SplitWs ws) {
     __shared__ ArgBest scratch[16];
     const int chunk = blockIdx.x, b = blockIdx.y;
+    if (seed_dev) {
+        seed_lo = seed_dev[0];
+        seed_hi = seed_dev[1];
+    }
     float v[4];
     int i0;
     split_load(logits + b * row_stride, V, chunk, v, i0);
@@ -379,12 +391,13 @@ extern "C" size_t gfa_sample_split_workspace(int n_rows, int V) {
 }
 
 // temperature <= 0 means greedy.  `workspace` has gfa_sample_split_workspace bytes; its
-// first n_rows * 1024 ints (the histograms) must be zero at the call.
-extern "C" int gfa_sample_split(const float* logits, size_t row_stride, int n_rows, int V,
-                                float temperature, int top_k, uint64_t seed, const int* row_keys,
-                                const int* positions, int position_offset, int* out,
-                                float* probs_out, void* workspace, hipStream_t stream) {
-    if (n_rows <= 0) return 0;
+// first n_rows * 1024 ints (the histograms) must be zero at the first call and are zero
+// again when a call has run, so one workspace serves call after call on one stream.
+// `seed_dev`: null, or two 32-bit words in device memory (low, high) that replace `seed`.
+static int run_sample_split(const float* logits, size_t row_stride, int n_rows, int V,
+                            float temperature, int top_k, uint64_t seed, const uint32_t* seed_dev,
+                            const int* row_keys, const int* positions, int position_offset,
+                            int* out, float* probs_out, void* workspace, hipStream_t stream) {
     SplitWs ws;
     ws.NB = (V + SPL_CHUNK - 1) / SPL_CHUNK;
     char* p = (char*)workspace;
@@ -409,7 +422,18 @@ extern "C" int gfa_sample_split(const float* logits, size_t row_stride, int n_ro
     split_sum_kernel<<<grid, SPL_THREADS, 0, stream>>>(logits, row_stride, V, t, use_pivot, ws);
     split_race_kernel<<<grid, SPL_THREADS, 0, stream>>>(
         logits, row_stride, V, t, use_pivot, (uint32_t)(seed & 0xffffffffu), (uint32_t)(seed >> 32),
-        row_keys, positions, position_offset, probs_out, ws);
+        seed_dev, row_keys, positions, position_offset, probs_out, ws);
     split_final_kernel<<<n_rows, 64, 0, stream>>>(out, ws);
     return GFA_LAUNCH_RESULT();
+}
+
+extern "C" int gfa_sample_split(const float* logits, size_t row_stride, int n_rows, int V,
+                                float temperature, int top_k, uint64_t seed,
+                                const uint32_t* seed_dev, const int* row_keys,
+                                const int* positions, int position_offset, int* out,
+                                float* probs_out, void* workspace, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (V <= 0 || !workspace) return (int)hipErrorInvalidValue;
+    return run_sample_split(logits, row_stride, n_rows, V, temperature, top_k, seed, seed_dev,
+                            row_keys, positions, position_offset, out, probs_out, workspace, stream);
 }

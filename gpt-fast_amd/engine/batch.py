@@ -6,12 +6,15 @@ its position, where that sequence's cache pages are) is laid out in one int32 bu
 that goes to the device in a single copy:
 
     tokens[N] tok_seq[N] tok_pos[N] q_start[B+1] start_pos[B] slots[B] row_keys[B]
-    want_rows[W] table_g[B, P_g] for every KV group g
+    want_rows[W] want_pos[W] seed[2] table_g[B, P_g] for every KV group g
 
 ``tok_seq[n]`` is the index of token n's sequence in this batch, ``tok_pos[n]`` its
 position in that sequence (tokens cached before the step + offset in the run);
 ``table_g[b, i]`` is the cache page that holds positions ``64 i .. 64 i + 63`` of
-sequence b in group g.
+sequence b in group g; ``want_rows`` are the indices of the tokens whose logits are wanted and
+``want_pos`` their positions; ``slots[b]`` is the sequence's slot, which indexes the fixed-size
+state of mixers that keep some; ``seed`` holds the two words of the sampler's seed for
+steps whose sampling is recorded and replayed.
 
 The reference's step takes ``idx[B, S]`` and one shared ``input_pos[S]`` (model.py:136)
 and a dense ``[Smax, Smax]`` mask (model.py:134); here lengths differ per sequence and
@@ -30,8 +33,9 @@ from ..cache.store import Cache, pages_for
 class Entry:
     """One sequence's share of a step: its slot, its new tokens, and the indices among
     these tokens whose logits are wanted.  ``slot`` None marks a row that belongs to no
-    sequence and only keeps a captured batch's shape: it reads and writes the cache's
-    spare page and its results are ignored."""
+    sequence and only keeps a recorded batch's shape: it reads and writes the cache's
+    spare page and spare state slot and its results are ignored.  Only a decode session
+    makes such rows; :meth:`Engine.step` refuses them."""
     slot: int
     tokens: Sequence[int]
     want: Sequence[int] = ()
@@ -52,7 +56,7 @@ class BatchLayout:
         self.fields = {}
         for name, count in (("tokens", n_tokens), ("tok_seq", n_tokens), ("tok_pos", n_tokens),
                             ("q_start", n_seqs + 1), ("start_pos", n_seqs), ("slots", n_seqs),
-                            ("row_keys", n_seqs), ("want_rows", n_want)):
+                            ("row_keys", n_seqs), ("want_rows", n_want), ("want_pos", n_want), ("seed", 2)):
             self.fields[name] = (off, count)
             off = _round_up(off + count, 4)          # 16-byte aligned fields
         self.tables = {}
@@ -99,9 +103,12 @@ class StepBatch:
 
 
 def fill_host(layout: BatchLayout, host: np.ndarray, entries: Sequence[Entry],
-              starts: Sequence[int], cache: Optional[Cache]) -> None:
+              starts: Sequence[int], cache: Optional[Cache], seed: int = 0) -> None:
     """Write the step's description into ``host`` (int32 of ``layout.size``)."""
+    from ..sampling import seed_words
     f = layout.fields
+    host[f["seed"][0]:f["seed"][0] + 2] = seed_words(seed)
+    spare_slot = cache.spare_slot if cache is not None else -1
     n = 0
     w = 0
     for b, (e, start) in enumerate(zip(entries, starts)):
@@ -114,12 +121,13 @@ def fill_host(layout: BatchLayout, host: np.ndarray, entries: Sequence[Entry],
         host[p0:p0 + q] = np.arange(start, start + q, dtype=np.int32)
         host[f["q_start"][0] + b] = n
         host[f["start_pos"][0] + b] = start
-        host[f["slots"][0] + b] = -1 if e.slot is None else e.slot
+        host[f["slots"][0] + b] = spare_slot if e.slot is None else e.slot
         host[f["row_keys"][0] + b] = e.key
         for i in e.want:
             if not 0 <= i < q:
                 raise ValueError(f"want index {i} is outside the {q} tokens of the entry")
             host[f["want_rows"][0] + w] = n + i
+            host[f["want_pos"][0] + w] = start + i
             w += 1
         n += q
     host[f["q_start"][0] + len(entries)] = n

@@ -4,7 +4,8 @@ generate.py:450-463, its driver at :272-437).
     python -m gpt_fast_amd --checkpoint_path MODEL_FOLDER --prompt "Hello, my name is"
     python -m gpt_fast_amd --random llama-3.1-8b --prompt 128 --batch_size 8
 
-``--checkpoint_path`` names a model *folder* (config.json + safetensors; the reference
+``--random`` takes a preset's name (of whichever registered architecture knows it, or of
+``--architecture``) or the path of a config.json.  ``--checkpoint_path`` names a model *folder* (config.json + safetensors; the reference
 takes a converted model.pth whose folder name selects the configuration,
 generate.py:222).  ``--prompt`` is text, or an integer N for a synthetic prompt of N
 random token ids below min(1024, vocabulary) as in generate.py:325-327.  Flags of the
@@ -13,6 +14,8 @@ compiled ahead of time) are accepted and ignored; those of features outside this
 library (--interactive, --speculate_k, --draft_checkpoint_path) are refused.
 """
 import argparse
+import json
+import os
 import sys
 import time
 from pathlib import Path
@@ -20,7 +23,7 @@ from typing import List, Optional, Union
 
 import torch
 
-from ..config.registry import architecture
+from ..config.registry import architecture_of, find_preset, read_model_folder
 from ..sampling import SamplingParams
 from .generate import generate
 from .step import Engine
@@ -50,7 +53,11 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--checkpoint_path", type=Path, default=None,
                    help="Model folder (config.json and safetensors files).")
     p.add_argument("--random", type=str, default=None, metavar="PRESET",
-                   help="Use seeded random weights of a named configuration instead of a folder.")
+                   help="Use seeded random weights of a named configuration (or of a "
+                        "config.json file) instead of a folder.")
+    p.add_argument("--architecture", type=str, default=None,
+                   help="Architecture whose preset --random names (default: the one that "
+                        "knows the name).")
     p.add_argument("--seed", type=int, default=1234, help="Seed of sampling and of --random.")
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--max_seq_length", type=int, default=None,
@@ -70,7 +77,7 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
          temperature: float = 0.8, checkpoint_path: Optional[Path] = None,
          random: Optional[str] = None, seed: int = 1234, dtype: str = "bfloat16",
          max_seq_length: Optional[int] = None, profile: Optional[Path] = None,
-         device: str = "cuda", out=print) -> dict:
+         device: str = "cuda", architecture_name: Optional[str] = None, out=print) -> dict:
     """Generates samples and reports throughput the way the reference's ``main`` does
     (generate.py:272-437).  Returns the aggregate numbers it printed."""
     if (checkpoint_path is None) == (random is None):
@@ -78,19 +85,35 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
     device = "cuda:0" if device == "cuda" else device
     out(f"Using device={device}")
 
+    # the model class and its configuration: by the folder's config.json, or by the preset's
+    # name among the registered architectures (or a config.json file given as the preset)
+    if checkpoint_path is not None:
+        arch, config = read_model_folder(str(checkpoint_path))
+    elif os.path.isfile(random):
+        with open(random) as f:
+            raw = json.load(f)
+        arch = architecture_of(raw)
+        config = arch.read_config(raw)
+    else:
+        arch, config = find_preset(random, architecture_name)
+
     tokenizer = None
     if isinstance(prompt, list):
         encoded = [int(t) for t in prompt]
     elif isinstance(prompt, int):
         encoded = None                       # synthetic, needs the vocabulary size
     else:
-        tokenizer = get_tokenizer(str(checkpoint_path)) if checkpoint_path else None
+        eos = getattr(config, "eos_token_id", None) or ()
+        tokenizer = get_tokenizer(str(checkpoint_path), bos=getattr(config, "bos_token_id", None),
+                                  eos=eos[0] if eos else None) if checkpoint_path else None
         if tokenizer is None:
             raise SystemExit("a text prompt needs a tokenizer.model or tokenizer.json in the "
                              "model folder (and sentencepiece or tokenizers); use an integer "
                              "--prompt for a synthetic prompt, or --prompt_ids")
-        encoded = encode_tokens(tokenizer, prompt, bos=True)
+        encoded = encode_tokens(tokenizer, prompt, bos=True)          # generate.py:213-217
     prompt_length = prompt if encoded is None else len(encoded)
+    if prompt_length < 1:
+        raise SystemExit("the prompt needs at least one token")
     per_seq = max_seq_length or (prompt_length + max_new_tokens)
     per_seq = (per_seq + 63) // 64 * 64
     if prompt_length + max_new_tokens > per_seq:
@@ -101,9 +124,8 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
     t0 = time.time()
     cache_args = dict(max_tokens=per_seq * batch_size, max_sequences=batch_size)
     if random is not None:
-        arch = architecture("llama")
-        engine = Engine.from_random("llama", arch.presets(random), seed, dtype=dtype,
-                                    device=device, **cache_args)
+        engine = Engine.from_random(arch.names[0], config, seed, dtype=dtype, device=device,
+                                    **cache_args)
     else:
         engine = Engine.from_folder(str(checkpoint_path), dtype=dtype, device=device, **cache_args)
     torch.cuda.synchronize()
@@ -114,6 +136,7 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
         hi = min(1024, engine.vocab_size)
         encoded = torch.randint(0, hi, (prompt,), generator=g).tolist()
     model_size = engine.model.parameter_bytes()
+    n_params = engine.model.parameter_count()
     tokens_per_sec = []
     result = None
     for i in range(-1, num_samples):                       # sample -1 warms up, generate.py:352
@@ -142,6 +165,9 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
         tokens_per_sec.append(tps)
         out(f"Time for inference {i + 1}: {t:.02f} sec total, {tps:.02f} tokens/sec")
         out(f"Bandwidth achieved: {model_size * tps / 1e9:.02f} GB/s")
+        # generate.py:421-424: every token of every sequence, prompt included, per second
+        total_tokens_sec = batch_size * len(seq) / t
+        out(f"FLOPS achieved: {n_params * total_tokens_sec * 2 / 1e12:.02f} TF/s")
         st = result.stats
         if st.get("decode_steps"):
             out(f"Decode: {st['decode_steps'] * batch_size / st['decode_seconds']:.02f} tokens/sec "
@@ -168,5 +194,5 @@ def cli(argv=None) -> int:
         prompt = [int(t) for t in args.prompt_ids.split(",")]
     main(prompt, args.num_samples, args.max_new_tokens, args.batch_size, args.top_k,
          args.temperature, args.checkpoint_path, args.random, args.seed, args.dtype,
-         args.max_seq_length, args.profile, args.device)
+         args.max_seq_length, args.profile, args.device, args.architecture)
     return 0

@@ -80,6 +80,12 @@ class BatchRun:
             [self.new[i][-1] for i in rows], self.max_new - 1)
         launched = {i: len(self.new[i]) for i in rows}       # tokens drawn or under way
         pending = None
+        try:
+            self._drive(session, rows, launched, pending)
+        finally:
+            session.close()
+
+    def _drive(self, session, rows, launched, pending) -> None:
         while True:
             active = [i for i in rows if self.reason[i] is None and launched[i] < self.max_new]
             handle = None
@@ -151,8 +157,7 @@ class EngineStepper:
         batch = self.engine.prepare(entries)
         logits = self.engine.model.forward(batch, self.engine.cache)
         # the drawn token sits one place after the last token of each entry
-        last_pos = batch.tok_pos.index_select(0, batch.want_rows.long())
-        tokens = sample(logits, self.params, batch.row_keys, last_pos, position_offset=1)
+        tokens = sample(logits, self.params, batch.row_keys, batch.want_pos, position_offset=1)
         out = tokens.tolist()
         dt = time.perf_counter() - t0
         if batch.is_decode:
@@ -187,6 +192,9 @@ class _TimedSession:
     def retire(self, row):
         self.session.retire(row)
 
+    def close(self):
+        self.session.close()
+
     def launch(self):
         if self.t_last is None:
             self.t_last = time.perf_counter()
@@ -210,6 +218,24 @@ def split_batches(n_requests: int, batch_size: Optional[int]) -> List[List[int]]
             for i in range(0, n_requests, batch_size)]
 
 
+def require_room(engine, prompts, max_new_tokens: int, batches) -> None:
+    """Before anything runs: every request stays within the model's positions (the
+    reference clamps its cache to them, generate.py:160-163) and every batch fits the cache
+    when all its requests have grown to their full length (the last token drawn is never
+    fed, so a request caches ``prompt + max_new_tokens - 1`` tokens)."""
+    plan = getattr(getattr(engine, "model", None), "plan", None)
+    most = getattr(plan, "max_positions", None)
+    for i, p in enumerate(prompts):
+        if most is not None and len(p) + max_new_tokens > most:
+            raise ValueError(f"request {i}: a prompt of {len(p)} tokens and {max_new_tokens} new "
+                             f"ones exceed the model's {most} positions")
+    cache = getattr(engine, "cache", None)
+    if cache is None:
+        return
+    for rows in batches:
+        cache.require_room([len(prompts[i]) + max_new_tokens - 1 for i in rows])
+
+
 def generate(engine, prompts: Sequence[Sequence[int]], max_new_tokens: int, *,
              temperature: float = 0.8, top_k: Optional[int] = None,
              stop_tokens: Optional[Sequence[int]] = None, seed: int = 1234,
@@ -229,11 +255,13 @@ def generate(engine, prompts: Sequence[Sequence[int]], max_new_tokens: int, *,
     if stop_tokens is None:
         stop_tokens = engine.model.plan.stop_tokens
     stepper = stepper or EngineStepper(engine, params, use_graph=use_graph)
+    batches = split_batches(len(prompts), batch_size)
+    require_room(engine, prompts, max_new_tokens, batches)
     tokens: List[List[int]] = [[] for _ in prompts]
     reasons: List[str] = ["length"] * len(prompts)
     steps = 0
     t0 = time.perf_counter()
-    for rows in split_batches(len(prompts), batch_size):
+    for rows in batches:
         cb = None
         if callback is not None:
             cb = (lambda r, t, rows=rows: callback([rows[i] for i in r], t))

@@ -19,6 +19,7 @@ from ..parts.model import DecoderModel
 from ..weights.bindings import compute_dtype, load_parameters
 from ..weights.random_init import random_parameters
 from .batch import BatchUploader, Entry, StepBatch
+from .decode import RecordedSteps
 
 
 def _device(device):
@@ -41,6 +42,7 @@ class Engine:
                            max_sequences=max_sequences, dtype=self.rt.dtype, device=self.rt.device)
         self.uploader = BatchUploader(self.rt.device)
         self.vocab_size = model.plan.vocab_size
+        self.recorded_steps = RecordedSteps(self)      # HIP graphs of the one-token step
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -84,6 +86,9 @@ class Engine:
             raise ValueError("a step needs at least one sequence")
         V = self.vocab_size
         for e in entries:
+            if e.slot is None:
+                raise ValueError("an entry without a slot is a filler row of a decode session; "
+                                 "a step takes sequences that hold a slot")
             if len(e.tokens) == 0:
                 raise ValueError(f"slot {e.slot}: a step brings at least one token per sequence")
             lo, hi = min(e.tokens), max(e.tokens)

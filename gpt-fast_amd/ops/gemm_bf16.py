@@ -152,15 +152,7 @@ def wide_f32_out(x: torch.Tensor, w: torch.Tensor):
     library with a float32 output; products of bfloat16 values are exact in float32 and
     the accumulation is float32."""
     require_device(x, w)
-    try:
-        return torch.mm(x, w.t(), out_dtype=torch.float32)
-    except (TypeError, RuntimeError):
-        out = torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
-        step = 8192
-        xf = x.float()
-        for n0 in range(0, w.shape[0], step):
-            out[:, n0:n0 + step] = xf @ w[n0:n0 + step].float().t()
-        return out
+    return torch.mm(x, w.t(), out_dtype=torch.float32)
 
 
 def qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages, n_heads: int,

@@ -221,6 +221,16 @@ def add_into(residual: torch.Tensor, y: torch.Tensor):
     return residual
 
 
+def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0):
+    """In place on float32 ``x``: x * scale, then cap * tanh(x / cap) if cap > 0."""
+    require_device(x)
+    require_contiguous(x=x)
+    _want(x, torch.float32, "x")
+    check(library("core").gfa_scale_cap(ptr(x), _sz(x.numel()), _f(scale), _f(cap),
+                                        stream_handle()), "scale_cap")
+    return x
+
+
 def add_rmsnorm(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float):
     """residual += float(y), then the RMS norm of the new rows in bfloat16: one pass.
     residual float32 [N, D], y bfloat16 [N, D], weight float32 [D]."""
@@ -243,21 +253,35 @@ def add_rmsnorm(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, e
 SPLIT_SAMPLING_ABOVE = 16384
 
 
+_split_workspaces = {}
+
+
 def _split_workspace(B: int, V: int, device) -> torch.Tensor:
-    lib = library("sampling")
-    lib.gfa_sample_split_workspace.restype = ctypes.c_size_t
-    n = lib.gfa_sample_split_workspace(_i(B), _i(V))
-    return torch.zeros(n // 4, dtype=torch.int32, device=device)      # histograms start at zero
+    """The workspace of the many-workgroup sampler for this many rows: allocated and zeroed
+    once per device and size; the kernels leave its histograms zero again, so it is used call
+    after call (on one stream at a time) and recorded launches keep a valid address."""
+    key = (torch.device(device).index, B, V)
+    ws = _split_workspaces.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("the sampler's workspace must exist before a step is recorded: "
+                              "run the step once outside the recording")
+        lib = library("sampling")
+        lib.gfa_sample_split_workspace.restype = ctypes.c_size_t
+        n = lib.gfa_sample_split_workspace(_i(B), _i(V))
+        ws = torch.zeros(n // 4, dtype=torch.int32, device=device)
+        _split_workspaces[key] = ws
+    return ws
 
 
-def _sample_split(logits, temperature, top_k, seed, row_keys, positions, position_offset, out,
-                  probs):
+def _sample_split(logits, temperature, top_k, seed, seed_words, row_keys, positions,
+                  position_offset, out, probs):
     B, V = logits.shape
     ws = _split_workspace(B, V, logits.device)
     check(library("sampling").gfa_sample_split(
         ptr(logits), _sz(logits.stride(0)), _i(B), _i(V), _f(temperature), _i(top_k),
-        ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(row_keys), ptr(positions), _i(position_offset),
-        ptr(out), ptr(probs), ptr(ws), stream_handle()), "sample_split")
+        ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(seed_words), ptr(row_keys), ptr(positions),
+        _i(position_offset), ptr(out), ptr(probs), ptr(ws), stream_handle()), "sample_split")
     return out
 
 
@@ -271,7 +295,7 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None):
     if out is None:
         out = torch.empty((B,), dtype=torch.int32, device=logits.device)
     if V > SPLIT_SAMPLING_ABOVE:
-        return _sample_split(logits, 0.0, 0, 0, None, None, 0, out, None)
+        return _sample_split(logits, 0.0, 0, 0, None, None, None, 0, out, None)
     check(library("sampling").gfa_argmax(ptr(logits), ptr(out), _i(B), _i(V),
                                          _sz(logits.stride(0)), stream_handle()), "argmax")
     return out
@@ -279,9 +303,15 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None):
 
 def sample(logits: torch.Tensor, temperature: float, top_k: Optional[int], seed: int,
            row_keys: torch.Tensor, positions: Optional[torch.Tensor], position_offset: int = 0,
-           out: Optional[torch.Tensor] = None, probs: Optional[torch.Tensor] = None):
-    """int32 [B]: one draw per row from softmax(top_k(logits / max(temperature, 1e-5)))."""
-    require_device(logits, row_keys, positions, probs)
+           out: Optional[torch.Tensor] = None, probs: Optional[torch.Tensor] = None,
+           seed_words: Optional[torch.Tensor] = None):
+    """int32 [B]: one draw per row from softmax(top_k(logits / max(temperature, 1e-5))).
+    ``seed_words``: int32 [2] on the device, the seed's low and high word; if given it
+    replaces ``seed`` (a recorded launch then follows the buffer's contents)."""
+    require_device(logits, row_keys, positions, probs, seed_words)
+    if seed_words is not None and (seed_words.dtype != torch.int32 or seed_words.numel() < 2
+                                   or not seed_words.is_contiguous()):
+        raise KernelError("sample: seed_words must be contiguous int32 [2]")
     _want(logits, torch.float32, "logits")
     _want(row_keys, torch.int32, "row_keys")
     if logits.dim() != 2 or logits.stride(1) != 1:
@@ -302,11 +332,11 @@ def sample(logits: torch.Tensor, temperature: float, top_k: Optional[int], seed:
     if V > SPLIT_SAMPLING_ABOVE:
         if temperature <= 0:
             raise KernelError("sample: temperature must be positive (greedy is argmax)")
-        return _sample_split(logits, temperature, k, seed, row_keys, positions, position_offset,
-                             out, probs)
+        return _sample_split(logits, temperature, k, seed, seed_words, row_keys, positions,
+                             position_offset, out, probs)
     check(library("sampling").gfa_sample(
         ptr(logits), _sz(logits.stride(0)), _i(B), _i(V), _f(temperature), _i(k),
-        ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(row_keys), ptr(positions),
+        ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(seed_words), ptr(row_keys), ptr(positions),
         _i(position_offset), ptr(out), ptr(probs), stream_handle()), "sample")
     return out
 

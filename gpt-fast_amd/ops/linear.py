@@ -54,12 +54,6 @@ class HalfNormed:
     def dtype(self):
         return self.xg.dtype
 
-    def materialize(self) -> torch.Tensor:
-        """The normed rows as an ordinary tensor (for a consumer that is no product here)."""
-        M, D = self.xg.shape
-        rs = torch.rsqrt(self.ssq.sum(dim=0)[:M, None] / D + self.eps)
-        return (self.xg.float() * rs).to(self.xg.dtype)
-
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
     """[M, N] = x [M, K] times w [N, K] transposed, in ``out_dtype`` (default: x's)."""

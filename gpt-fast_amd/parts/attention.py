@@ -39,6 +39,10 @@ class Attention(Part):
         s = self.spec
         return KVNeed(s.n_kv_heads, s.head_dim, s.window)
 
+    @property
+    def replayable(self):
+        return bool(getattr(self.position, "replayable", False))
+
     prepares_norm = True
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 

@@ -18,6 +18,12 @@ Interfaces (N = tokens of the step, D = model width):
 A new part is a class with these methods, registered under a new ``kind``; its spec is
 any object with that ``kind`` attribute.
 
+``replayable = True`` on a part says that its ``forward`` issues the same kernels, with
+the same arguments, whatever the batch holds - it reads the batch's device fields only,
+never ``host_field`` or a host copy - so that a step recorded once can be replayed for
+later steps of the same shape.  A part without it (the default) makes generation step the
+model without a recording.
+
 Optional, for speed only: a mixer or feed-forward that sets ``prepares_norm = True`` also
 takes ``then_norm=`` (the norm that reads the residual stream after it) and
 ``takes_halves=`` and returns that norm's rows if its last kernel produced them on the way,
@@ -58,6 +64,8 @@ class Runtime:
 
 
 class Part:
+    replayable = False
+
     def parameters(self) -> Dict[str, Param]:
         return {}
 

@@ -47,6 +47,10 @@ class PreNormBlock(Part):
     prepares_norm = True
 
     @property
+    def replayable(self):
+        return all(getattr(c, "replayable", False) for c in self.children().values())
+
+    @property
     def takes_prepared(self):
         return getattr(self.mixer, "takes_prepared", False)
 

@@ -23,6 +23,7 @@ class GatedFeedForward(Part):
         check_bound("GatedFeedForward", self.parameters(), tensors)
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
+    replayable = True
     prepares_norm = True
     # x may be an ops.linear.HalfNormed, from one row on (the least number of rows; with the
     # weights streamed past the caches the matrix-core kernel that takes the halves is as fast

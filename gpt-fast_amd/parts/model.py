@@ -6,11 +6,13 @@ import torch
 from ..config.spec import ModelPlan
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import BLOCKS, NORMS, Param, Runtime, check_bound
+from .base import BLOCKS, NORMS, POSITIONS, Param, Runtime, check_bound
 
 
 class DecoderModel:
-    """Embedding, the plan's layers in the plan's order, final norm, output head.
+    """Embedding, the plan's layers in the plan's order, final norm, output head; around
+    them the optional steps a plan may state (a factor on the embedded rows, a position
+    encoding added to them, a factor and a soft cap on the logits).
 
     ``forward`` runs the tokens of one step: embeds them, passes the float32 residual
     stream through every run of the order with that run's cache entry, then norms and
@@ -23,6 +25,12 @@ class DecoderModel:
         self.rt = runtime
         self.blocks = [BLOCKS.build(_Arranged(layer), runtime) for layer in plan.layers]
         self.final_norm = NORMS.build(plan.final_norm, runtime)
+        self.input_position = None
+        if plan.input_position is not None:
+            self.input_position = POSITIONS.build(plan.input_position, runtime)
+            if not hasattr(self.input_position, "add_to_stream"):
+                raise TypeError(f"position kind '{plan.input_position.kind}' cannot be a plan's "
+                                f"input_position: its part has no add_to_stream(residual, batch)")
         self.embedding = self.head = None
 
     # ------------------------------------------------------------------ parameters
@@ -30,6 +38,9 @@ class DecoderModel:
         p = {self.plan.embedding_name: Param((self.plan.vocab_size, self.plan.dim)),
              self.plan.head_name: Param((self.plan.vocab_size, self.plan.dim)),
              self.plan.final_norm_name: Param((self.plan.dim,), "vector", "norm")}
+        if self.input_position is not None:
+            for name, param in self.input_position.parameters().items():
+                p[f"{self.plan.input_position_name}.{name}"] = param
         for layer, block in zip(self.plan.layers, self.blocks):
             for name, param in block.parameters().items():
                 p[f"{layer.name}.{name}"] = param
@@ -45,6 +56,10 @@ class DecoderModel:
         self.embedding = tensors[self.plan.embedding_name]
         self.head = tensors[self.plan.head_name]
         self.final_norm.bind({"weight": tensors[self.plan.final_norm_name]})
+        if self.input_position is not None:
+            prefix = self.plan.input_position_name + "."
+            self.input_position.bind({k[len(prefix):]: v for k, v in tensors.items()
+                                      if k.startswith(prefix)})
         for layer, block in zip(self.plan.layers, self.blocks):
             prefix = layer.name + "."
             block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
@@ -62,6 +77,28 @@ class DecoderModel:
                 total += t.numel() * t.element_size()
         return total
 
+    @property
+    def replayable(self) -> bool:
+        """Every part issues the same kernels whatever a batch holds: a recorded step can be
+        replayed."""
+        return (all(getattr(b, "replayable", False) for b in self.blocks)
+                and getattr(self.final_norm, "replayable", False)
+                and (self.input_position is None
+                     or getattr(self.input_position, "replayable", False)))
+
+    def parameter_count(self, exclude_embedding: bool = True) -> int:
+        """Elements of the same parameters (the reference's ``params`` of
+        generate.py:251-268, which feeds its FLOPS line)."""
+        seen, total = set(), 0
+        for name, t in self._tensors.items():
+            if exclude_embedding and name == self.plan.embedding_name \
+                    and t.data_ptr() != self.head.data_ptr():
+                continue
+            if t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel()
+        return total
+
     # ------------------------------------------------------------------ cache
     def cache_needs(self) -> List[object]:
         return [self.blocks[run.layer].cache_need() for run in self.plan.order]
@@ -72,8 +109,13 @@ class DecoderModel:
     # ------------------------------------------------------------------ step
     def forward(self, batch, cache) -> torch.Tensor:
         """float32 logits [n_wanted, vocab] of the step described by ``batch``."""
+        plan = self.plan
         residual = K.embed(self.embedding, batch.tokens)                  # model.py:140
-        order = self.plan.order
+        if plan.embedding_scale is not None:
+            K.scale_cap(residual, plan.embedding_scale)
+        if self.input_position is not None:
+            self.input_position.add_to_stream(residual, batch)
+        order = plan.order
         x = None                       # rows of the next norm, if a block produced them
         for n, run in enumerate(order):                                   # model.py:142-143
             block = self.blocks[run.layer]
@@ -98,7 +140,11 @@ class DecoderModel:
                                device=residual.device)
         if x is None:
             x = self.final_norm.forward(residual, rows=batch.want_rows)   # model.py:144
-        return L.linear(x, self.head, out_dtype=torch.float32)            # model.py:145
+        logits = L.linear(x, self.head, out_dtype=torch.float32)          # model.py:145
+        if plan.logit_scale is not None or plan.logit_softcap is not None:
+            K.scale_cap(logits, 1.0 if plan.logit_scale is None else plan.logit_scale,
+                        plan.logit_softcap or 0.0)
+        return logits
 
 
 class _Arranged:

@@ -11,6 +11,8 @@ class RMSNorm(Part):
     scaling in float32 from the float32 residual stream, one rounding to the compute type
     at the store.  ``eps`` and the width are the spec's."""
 
+    replayable = True
+
     def __init__(self, spec: NormSpec, runtime: Runtime):
         self.spec = spec
         self.rt = runtime

@@ -43,6 +43,7 @@ FREQUENCY_SCALINGS = {"llama3": llama3_scaled}
 
 class RotaryPosition(Part):
     LAYOUTS = {"interleaved": 0, "half": 1}
+    replayable = True
 
     def __init__(self, spec: PositionSpec, runtime: Runtime):
         if spec.layout not in self.LAYOUTS:
@@ -85,6 +86,7 @@ class RotaryPosition(Part):
 
 class NoPosition(Part):
     """No position information: q, k, v pass through unchanged into q and the cache."""
+    replayable = True
 
     def __init__(self, spec: PositionSpec, runtime: Runtime):
         self.spec = spec

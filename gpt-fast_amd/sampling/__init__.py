@@ -34,10 +34,13 @@ class SamplingParams:
 
 def sample(logits: torch.Tensor, params: SamplingParams, row_keys: torch.Tensor,
            positions: Optional[torch.Tensor], position_offset: int = 0,
-           out: Optional[torch.Tensor] = None, probs: Optional[torch.Tensor] = None):
+           out: Optional[torch.Tensor] = None, probs: Optional[torch.Tensor] = None,
+           seed_words: Optional[torch.Tensor] = None):
     """int32 [B] next tokens for float32 logits [B, V].  ``row_keys`` (int32 [B])
     identifies each row's request and ``positions`` (+ offset) the place of the token
-    being drawn; both only feed the noise."""
+    being drawn; both only feed the noise.  ``seed_words`` (int32 [2] on the device: the
+    seed's low and high word) replaces ``params.seed`` where the launch is recorded and
+    replayed for other seeds."""
     if params.greedy and probs is None:
         return K.argmax(logits, out=out)
     if params.greedy:
@@ -46,7 +49,15 @@ def sample(logits: torch.Tensor, params: SamplingParams, row_keys: torch.Tensor,
                  position_offset, out=None, probs=probs)
         return K.argmax(logits, out=out)
     return K.sample(logits, params.temperature, params.top_k, params.seed, row_keys,
-                    positions, position_offset, out=out, probs=probs)
+                    positions, position_offset, out=out, probs=probs, seed_words=seed_words)
+
+
+def seed_words(seed: int):
+    """The low and high 32-bit word of a seed as the signed integers an int32 buffer holds."""
+    def signed(u):
+        return u - (1 << 32) if u >= (1 << 31) else u
+    seed &= (1 << 64) - 1
+    return signed(seed & 0xFFFFFFFF), signed(seed >> 32)
 
 
 def logits_to_probs(logits: torch.Tensor, temperature: float = 1.0,

@@ -5,7 +5,8 @@ its plan (:class:`Binding`); this module finds the tensors, checks all names and
 in one pass and reports every problem in a single :class:`WeightsError`, then builds
 the parameters on the device.
 
-Dtype rule.  ``role`` says how a parameter is used: a "matrix" (operand of a matrix
+Dtype rule.  ``role`` says how a parameter is used (the table ``ROLES``, open to further
+roles through :func:`register_role`): a "matrix" (operand of a matrix
 product, also the embedding table) is kept in the engine's compute type (bfloat16 or
 float32); a "vector" (norm weights and the like) is kept in float32, which holds a
 bfloat16 value exactly; an "index" table is int32.  A tensor stored in 32-bit is never
@@ -79,14 +80,26 @@ def compute_dtype(name) -> torch.dtype:
     raise ValueError(f"dtype '{name}': bfloat16 or float32")
 
 
+# role -> (storage type given the engine's compute type, whether the stored tensor must be
+# of a floating type)
+ROLES: Dict[str, Tuple[Callable[[torch.dtype], torch.dtype], bool]] = {
+    "matrix": (lambda dtype: dtype, True),
+    "vector": (lambda dtype: torch.float32, True),
+    "index": (lambda dtype: torch.int32, False),
+}
+
+
+def register_role(role: str, storage: Callable[[torch.dtype], torch.dtype],
+                  floating: bool = True) -> None:
+    """A further way a parameter is used (a state-space model's float32 recurrence
+    matrices, say): ``storage(compute type)`` is the type it is kept in."""
+    ROLES[role] = (storage, floating)
+
+
 def dtype_for_role(role: str, dtype: torch.dtype) -> torch.dtype:
-    if role == "matrix":
-        return dtype
-    if role == "vector":
-        return torch.float32
-    if role == "index":
-        return torch.int32
-    raise ValueError(f"unknown parameter role '{role}'")
+    if role not in ROLES:
+        raise ValueError(f"unknown parameter role '{role}'; known: {sorted(ROLES)}")
+    return ROLES[role][0](dtype)
 
 
 def check_layout(layout: CheckpointLayout, entries: Dict[str, Tuple[str, tuple]], where: str):
@@ -108,7 +121,7 @@ def check_layout(layout: CheckpointLayout, entries: Dict[str, Tuple[str, tuple]]
             dt, shape = entries[s.name]
             if tuple(shape) != tuple(s.shape):
                 wrong.append((s.name, tuple(shape), tuple(s.shape)))
-            if b.role in ("matrix", "vector") and dt not in ("F64", "F32", "F16", "BF16"):
+            if ROLES.get(b.role, (None, True))[1] and dt not in ("F64", "F32", "F16", "BF16"):
                 other.append(f"{s.name} is stored as {dt}, expected a floating type")
     ignored = [re.compile(p) for p in layout.ignored]
     unexpected = [n for n in entries

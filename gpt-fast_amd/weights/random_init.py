@@ -20,16 +20,28 @@ def _tensor_seed(seed: int, name: str) -> int:
     return (int(seed) * 1000003 + zlib.crc32(name.encode("utf-8"))) % (2 ** 63 - 1)
 
 
+# init name -> function(standard normal float32 tensor, std, norm_std) -> tensor
+INITS = {
+    "linear": lambda t, std, norm_std: t.mul_(std),                    # N(0, std)
+    "norm": lambda t, std, norm_std: t.mul_(norm_std).add_(1.0),       # 1 + N(0, norm_std)
+}
+
+
+def register_init(name: str, fn) -> None:
+    """A further law for random weights: ``fn(t, std, norm_std)`` maps a tensor of standard
+    normal draws of the parameter's shape to the parameter (a decay rate kept in (0, 1), a
+    table of integers, ...)."""
+    INITS[name] = fn
+
+
 def draw(source, seed: int, device, std: float, norm_std: float) -> torch.Tensor:
-    """One checkpoint tensor in float32: "linear" N(0, std), "norm" 1 + N(0, norm_std)."""
+    """One checkpoint tensor in float32, by the law its ``init`` names in ``INITS``."""
+    if source.init not in INITS:
+        raise ValueError(f"unknown init '{source.init}' for {source.name}; known: {sorted(INITS)}")
     g = torch.Generator(device=device)
     g.manual_seed(_tensor_seed(seed, source.name))
     t = torch.randn(source.shape, generator=g, device=device, dtype=torch.float32)
-    if source.init == "linear":
-        return t.mul_(std)
-    if source.init == "norm":
-        return t.mul_(norm_std).add_(1.0)
-    raise ValueError(f"unknown init '{source.init}' for {source.name}")
+    return INITS[source.init](t, std, norm_std)
 
 
 def random_checkpoint(layout: CheckpointLayout, seed: int, dtype="bfloat16", *,

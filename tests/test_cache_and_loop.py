@@ -56,7 +56,8 @@ def test_groups_by_need():
     assert (c.entries[0].index, c.entries[2].index) == (0, 1)
     assert c.groups[c.entries[0].group_id].k.shape == (2, 7, 2, 64, 8)       # 6 pages and the spare one
     assert c.groups[c.entries[0].group_id].v.shape == (2, 7, 2, 8, 64)
-    assert c.entries[3].state.shape == (4, 3)
+    assert c.entries[3].state.shape == (5, 3)                  # 4 slots and the spare one
+    assert c.spare_slot == 4
     # a borrowed entry reads the lender's storage and does not write
     b = Cache([KVNeed(1, 8), KVNeed(1, 8)], [None, 0], max_tokens=64, max_sequences=1,
               dtype=torch.float32, device="cpu")
@@ -143,12 +144,74 @@ def test_batch_description_layout():
     assert list(f("tok_seq")[:4]) == [0, 0, 0, 1] and list(f("tok_pos")[:5]) == [0, 1, 2, 0, 1]
     assert list(f("q_start")) == [0, 3, 73] and list(f("want_rows")) == [0, 2, 72]
     assert list(f("row_keys")) == [11, 12]
+    assert list(f("want_pos")) == [0, 2, 69] and list(f("slots")) == [a, b]
+    assert list(f("seed")) == [0, 0]
     off, n = lay.tables[0]
     table = host[off:off + n].reshape(2, 2)
     assert table[0, 0] == c.page_list(0, a)[0] and table[0, 1] == -1
     assert list(table[1]) == c.page_list(0, b)
     with pytest.raises(ValueError):
         fill_host(lay, host, [Entry(a, [1, 2, 3], want=[3]), entries[1]], starts, c)
+
+
+def test_filler_rows_point_at_the_spare_page_and_slot_and_the_seed_is_two_words():
+    c = make_cache()
+    a = c.acquire()
+    starts = c.extend_many([(a, 1)]) + [0]
+    entries = [Entry(a, [5], want=[0], key=1), Entry(None, [0], want=[0], key=2)]
+    lay = BatchLayout(2, 2, 2, {gid: 3 for gid, _ in c.kv_groups})
+    host = np.zeros(lay.size, dtype=np.int32)
+    fill_host(lay, host, entries, starts, c, seed=(5 << 32) | 0xFFFFFFFE)
+    f = lambda name: host[lay.fields[name][0]: lay.fields[name][0] + lay.fields[name][1]]
+    assert list(f("slots")) == [a, c.spare_slot] and c.spare_slot == c.max_sequences
+    assert list(f("seed")) == [-2, 5]                 # low word 0xFFFFFFFE as int32, high word
+    for gid, g in c.kv_groups:
+        off, n = lay.tables[gid]
+        table = host[off:off + n].reshape(2, 3)
+        assert list(table[1]) == [g.spare_page] * 3 and table[0, 0] == c.page_list(gid, a)[0]
+    # the spare slot's state is nobody's: acquiring every slot never hands it out
+    held = [a] + [c.acquire() for _ in range(c.max_sequences - 1)]
+    assert c.spare_slot not in held
+    with pytest.raises(CacheFull):
+        c.acquire()
+
+
+def test_room_is_checked_for_whole_batches():
+    c = make_cache(max_tokens=64 * 6, max_sequences=4)
+    c.require_room([64, 64, 128, 100])                # 1 + 1 + 2 + 2 pages
+    with pytest.raises(CacheFull, match="tokens"):
+        c.require_room([65, 64, 128, 100])
+    with pytest.raises(CacheFull, match="slots"):
+        c.require_room([1, 1, 1, 1, 1])
+
+
+def test_generate_refuses_before_it_starts():
+    """Too long for the model's positions, or too much for the cache: an error before any
+    slot is taken or any step runs."""
+    class Plan:
+        stop_tokens = ()
+        max_positions = 50
+
+    class Model:
+        plan = Plan
+
+    class Eng:
+        model = Model
+        cache = make_cache(max_tokens=64 * 2, max_sequences=2)
+
+    st = ScriptedStepper(lambda key, fed: 1)
+    with pytest.raises(ValueError, match="50 positions"):
+        generate(Eng, [[1] * 45], 6, temperature=0.0, stepper=st)
+    Plan.max_positions = 200
+    with pytest.raises(CacheFull):
+        generate(Eng, [[1] * 30, [2] * 30, [3]], 5, temperature=0.0, stepper=st)
+    with pytest.raises(CacheFull):                    # 70 tokens each: two pages each
+        generate(Eng, [[1] * 40] * 2, 31, temperature=0.0, stepper=st, batch_size=2)
+    assert st.calls == [] and st.slots.held == 0
+    # the last token drawn is never fed: 60 + 5 - 1 = 64 tokens are one page each
+    Plan.max_positions = 65
+    out = generate(Eng, [[1] * 60, [2] * 60], 5, temperature=0.0, stepper=st)
+    assert [len(t) for t in out.tokens] == [5, 5]
 
 
 class ScriptedStepper:
@@ -261,6 +324,9 @@ class SessionStepper(ScriptedStepper):
 
             def collect(self, handle):
                 return handle
+
+            def close(self):
+                self.closed = True
         self.session = Session()
         return self.session
 
@@ -277,6 +343,7 @@ def test_loop_with_a_session_notices_stops_one_step_late():
     # request 3 ended in the prefill and never entered the session; requests 0 and 2 end
     # by length and are not launched beyond it: 4 decode steps in all
     assert len(st.session.slots) == 3 and st.session.launches == 4
+    assert st.session.closed
     # request 1's filler row was retired after its stop token was seen
     assert st.session.slots == [0, None, 2] or st.session.slots[1] is None
 

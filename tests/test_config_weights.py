@@ -236,3 +236,90 @@ def test_random_model_is_seeded_and_sharded_index_is_read(tmp_path):
     p1 = load_parameters(sh, arch.bindings(c2), "float32", None)
     p0 = load_parameters(a, arch.bindings(c2), "float32", None)
     assert all(torch.equal(p0[k], p1[k]) for k in p0)
+
+
+def test_presets_are_found_through_the_registry():
+    from gpt_fast_amd.config.registry import find_preset
+    arch, cfg = find_preset("llama-3.1-8b")
+    assert arch is gfa.architecture("llama") and cfg.hidden_size == 4096
+    arch, cfg = find_preset("tiny-llama-b", "LlamaForCausalLM")
+    assert cfg.num_key_value_heads == 2
+    with pytest.raises(UnknownArchitecture, match="preset"):
+        find_preset("no-such-model")
+    with pytest.raises(UnknownArchitecture):
+        find_preset("7B", "no-such-architecture")
+
+
+def test_roles_and_inits_are_open_tables(tmp_path):
+    """A parameter of a further kind - kept in float32 whatever the engine computes in,
+    drawn from a law of its own - needs an entry in two tables and no change to the
+    loader or to the random-weights mode."""
+    from gpt_fast_amd.weights import bindings as B
+    from gpt_fast_amd.weights import random_init as R
+    B.register_role("toy_decay", lambda dtype: torch.float32)
+    R.register_init("toy_unit_interval", lambda t, std, norm_std: torch.sigmoid(t))
+    try:
+        layout = B.CheckpointLayout((
+            B.Binding("decay", (B.Source("blk.decay", (5, 3), "toy_unit_interval"),), role="toy_decay"),
+            B.Binding("mix", (B.Source("blk.mix", (4, 4)),)),
+        ))
+        ck = R.random_checkpoint(layout, seed=1, dtype="bfloat16")
+        assert ck["blk.decay"].min() > 0 and ck["blk.decay"].max() < 1
+        write_safetensors(str(tmp_path / "model.safetensors"),
+                          {"blk.decay": ck["blk.decay"].float(), "blk.mix": ck["blk.mix"]})
+        params = load_parameters(str(tmp_path), layout, "bfloat16", None)
+        assert params["decay"].dtype == torch.float32 and params["mix"].dtype == torch.bfloat16
+        drawn = R.random_parameters(layout, 1, "bfloat16", "cpu")
+        assert drawn["decay"].dtype == torch.float32
+    finally:
+        del B.ROLES["toy_decay"], R.INITS["toy_unit_interval"]
+    with pytest.raises(ValueError, match="role"):
+        B.dtype_for_role("toy_decay", torch.bfloat16)
+    with pytest.raises(ValueError, match="init"):
+        R.draw(B.Source("x", (2,), "toy_unit_interval"), 0, "cpu", 0.02, 0.1)
+
+
+def test_text_prompts_start_with_bos(tmp_path):
+    """generate.py:213-217: the BOS id goes in front.  A tokenizer.json has no BOS id of its
+    own; it comes from the model's configuration."""
+    from gpt_fast_amd.engine.tokenizer import Tokenizer, encode_tokens, get_tokenizer
+
+    class Stub(Tokenizer):
+        def encode(self, text):
+            return [len(w) for w in text.split()]
+
+        def bos_id(self):
+            return 99
+
+    assert encode_tokens(Stub(), "a bb ccc") == [99, 1, 2, 3]
+    assert encode_tokens(Stub(), "a bb", bos=False) == [1, 2]
+    tokenizers = pytest.importorskip("tokenizers")
+    tk = tokenizers.Tokenizer(tokenizers.models.WordLevel({"w0": 0, "w1": 1, "w2": 2}, unk_token="w0"))
+    tk.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tk.save(str(tmp_path / "tokenizer.json"))
+    t = get_tokenizer(str(tmp_path), bos=7, eos=8)
+    assert encode_tokens(t, "w2 w1") == [7, 2, 1] and t.eos_id() == 8
+    assert encode_tokens(get_tokenizer(str(tmp_path)), "w2 w1") == [2, 1]    # no id known: none added
+
+
+def test_a_library_is_rebuilt_when_its_source_changes(tmp_path, monkeypatch):
+    """The stamp beside a built library holds a hash of source, common header and flags; a
+    library whose stamp does not fit is not current."""
+    from gpt_fast_amd.csrc import build as b
+    (tmp_path / "toy.hip").write_text("// one\n")
+    (tmp_path / "common.h").write_text("// header\n")
+    monkeypatch.setattr(b, "HERE", str(tmp_path))
+    lib = tmp_path / "libgfa_toy.so"
+    assert not b._is_current(str(lib), "toy")                       # nothing built
+    lib.write_text("binary")
+    assert not b._is_current(str(lib), "toy")                       # no stamp
+    (tmp_path / "libgfa_toy.so.stamp").write_text(b.source_hash("toy"))
+    assert b._is_current(str(lib), "toy")
+    (tmp_path / "toy.hip").write_text("// two\n")
+    assert not b._is_current(str(lib), "toy")                       # source edited
+    (tmp_path / "libgfa_toy.so.stamp").write_text(b.source_hash("toy"))
+    (tmp_path / "common.h").write_text("// header, edited\n")
+    assert not b._is_current(str(lib), "toy")                       # header edited
+    (tmp_path / "libgfa_toy.so.stamp").write_text(b.source_hash("toy"))
+    monkeypatch.setattr(b, "FLAGS", b.FLAGS + ["-DX"])
+    assert not b._is_current(str(lib), "toy")                       # flags changed

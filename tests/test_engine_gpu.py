@@ -132,3 +132,98 @@ def test_batch_of_forty_shrinking_to_one(tmp_path_factory, name, dtype, tol):
         assert rel_err(torch.cat(got[i]), want) < tol, (name, dtype, i)
     eng.cache.check()
     assert eng.cache.slots.held == 0
+
+
+# --------------------------------------------------------------------------------------
+# Steps of several tokens at a position other than 0 (the reference runs such a step when it
+# verifies a draft, generate.py:104-108, and its mask row is chosen by input_pos,
+# model.py:138), and steps that hold rows of every kind at once.
+def _chunked(eng, tokens, cuts):
+    """Feed ``tokens`` of one sequence as chunks of the given sizes; logits of every row."""
+    from gpt_fast_amd import Entry
+    assert sum(cuts) == len(tokens)
+    slot = eng.start_sequence()
+    got, at = [], 0
+    for n in cuts:
+        got.append(eng.step([Entry(slot, tokens[at:at + n], want=list(range(n)))]).cpu())
+        at += n
+    eng.end_sequence(slot)
+    return torch.cat(got)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_chunks_at_offsets_off_the_page_edges(tmp_path_factory, name, dtype, tol):
+    """100 tokens as chunks of 37 + 29 + 1 + 33: every chunk after the first starts at a
+    position that is neither 0 nor a multiple of the page size, and the second ends inside
+    the second page."""
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype)
+    V = util.TINY[name]["vocab_size"]
+    tokens = util.random_tokens(V, 100, 21)
+    want = util.plain_logits(folder, tokens)
+    got = _chunked(eng, tokens, [37, 29, 1, 33])
+    assert rel_err(got, want) < tol
+    if dtype == "float32":
+        assert torch.equal(got, whole(eng, tokens))
+    # other cuts, among them chunks that end exactly on a page edge and one-token chunks
+    for cuts in ([64, 36], [63, 1, 36], [1, 1, 62, 36], [5, 95]):
+        g2 = _chunked(eng, tokens, cuts)
+        assert rel_err(g2, want) < tol, cuts
+        if dtype == "float32":
+            assert torch.equal(g2, got), cuts
+    eng.cache.check()
+    assert eng.cache.slots.held == 0
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_one_step_with_decode_rows_a_chunk_and_a_fresh_prompt(tmp_path_factory, name, dtype, tol):
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), name, dtype="float32")
+    eng = engine_for(folder, dtype)
+    V = util.TINY[name]["vocab_size"]
+    seqs, before, mixed = util.mixed_step_case(V)
+    slots = {r: eng.start_sequence() for r in seqs}
+    got = {r: [] for r in seqs}
+    order = ["d0", "d1", "d2", "c"]
+    logits = eng.step([Entry(slots[r], seqs[r][:before[r]], want=list(range(before[r])))
+                       for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + before[r]])
+        at += before[r]
+    # the mixed step, rows in an order that puts the chunk between single tokens
+    order = ["d0", "c", "d1", "p", "d2"]
+    fed = {r: before.get(r, 0) for r in order}
+    logits = eng.step([Entry(slots[r], seqs[r][fed[r]:fed[r] + mixed[r]],
+                             want=list(range(mixed[r]))) for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + mixed[r]])
+        at += mixed[r]
+        fed[r] += mixed[r]
+    # the rest of the chunked sequence and of the prompt, one token each, together
+    for r in ("c", "p"):
+        while fed[r] < len(seqs[r]):
+            got[r].append(eng.step([Entry(slots[r], [seqs[r][fed[r]]], want=[0])]).cpu())
+            fed[r] += 1
+    for r, toks in seqs.items():
+        want = util.plain_logits(folder, toks)
+        g = torch.cat(got[r])
+        assert g.shape == want.shape
+        assert rel_err(g, want) < tol, (name, dtype, r)
+        if dtype == "float32":
+            assert torch.equal(g, whole(eng, toks)), (name, r)
+        eng.end_sequence(slots[r])
+    eng.cache.check()
+    assert eng.cache.slots.held == 0
+
+
+def test_a_step_refuses_rows_without_a_slot(tmp_path_factory):
+    from gpt_fast_amd import Entry
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "A", dtype="float32")
+    eng = engine_for(folder, "float32")
+    with pytest.raises(ValueError, match="filler"):
+        eng.step([Entry(None, [1, 2], want=[1])])
+    assert eng.cache.slots.held == 0

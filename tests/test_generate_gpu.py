@@ -267,92 +267,6 @@ def test_parts_alone(tmp_path_factory):
     assert rel_err(res, want) < 1e-5
 
 
-def test_toy_mixer_with_state_registers_and_steps(tmp_path_factory):
-    """A mixer defined here, with fixed-size state per sequence and no keys or values, is
-    registered, built into a plan next to attention layers, and stepped: no file of the
-    library changes.  It computes a running mean of its inputs (state: sum and count),
-    which the plain check below recomputes from the whole sequence."""
-    from dataclasses import dataclass
-    import gpt_fast_amd as gfa
-    from gpt_fast_amd import Entry
-    from gpt_fast_amd.cache.store import StateNeed
-    from gpt_fast_amd.config.spec import LayerSpec, ModelPlan, NormSpec, Run
-    from gpt_fast_amd.parts import Param, Part, register_mixer
-
-    @dataclass(frozen=True)
-    class RunningMeanSpec:
-        dim: int
-        kind: str = "toy_running_mean"
-
-    class RunningMean(Part):
-        def __init__(self, spec, rt):
-            self.spec, self.rt = spec, rt
-
-        def parameters(self):
-            return {"mix": Param((self.spec.dim, self.spec.dim))}
-
-        def bind(self, tensors):
-            self.mix = tensors["mix"]
-
-        def cache_need(self):
-            return StateNeed((self.spec.dim + 1,), "float32")
-
-        def forward(self, x, batch, entry, residual):
-            state = entry.state                                   # [n_slots, dim + 1]
-            q_start = batch.host_field("q_start")
-            slots = batch.host_field("slots")
-            for b in range(batch.n_seqs):
-                lo, hi = int(q_start[b]), int(q_start[b + 1])
-                xs = x[lo:hi].float()
-                s = state[int(slots[b])]
-                sums = s[:-1] + torch.cumsum(xs, 0)
-                counts = s[-1] + torch.arange(1, hi - lo + 1, device=x.device)
-                residual[lo:hi] += (sums / counts[:, None]) @ self.mix.float().T
-                s[:-1] = sums[-1]
-                s[-1] = counts[-1]
-
-    register_mixer("toy_running_mean", RunningMean)
-
-    arch = gfa.architecture("llama")
-    cfg = arch.read_config(util.TINY_A)
-    base = arch.plan(cfg)
-    D = cfg.hidden_size
-    toy_layer = LayerSpec(name="toy", mixer=RunningMeanSpec(D), mixer_norm=NormSpec(D, 1e-5),
-                          feed_forward=base.layers[0].feed_forward,
-                          feed_forward_norm=NormSpec(D, 1e-5))
-    # attention, toy, attention again with the first run's weights *and* cache (borrowed)
-    plan = ModelPlan(dim=D, vocab_size=cfg.vocab_size,
-                     layers=[base.layers[0], toy_layer, base.layers[1]],
-                     order=[Run(0), Run(1), Run(2), Run(1), Run(0, cache_from=0)],
-                     final_norm=base.final_norm)
-    from gpt_fast_amd.parts import Runtime
-    from gpt_fast_amd.parts.model import DecoderModel
-    model = DecoderModel(plan, Runtime(torch.float32, "cuda:0"))
-    g = torch.Generator().manual_seed(0)
-    params = {}
-    for name, p in model.parameters().items():
-        t = torch.randn(p.shape, generator=g) * 0.05
-        params[name] = (1 + t if p.init == "norm" else t).to("cuda:0")
-    eng = gfa.Engine.from_plan(plan, params, "float32", "cuda:0", max_tokens=512)
-    assert len(eng.cache.groups) == 2             # one KV group, one state group of two entries
-    toks = util.random_tokens(cfg.vocab_size, 90, 3)
-    slot = eng.start_sequence()
-    whole = eng.step([Entry(slot, toks, want=list(range(90)))]).cpu()
-    eng.end_sequence(slot)
-    # the same tokens cut into a prompt and single tokens, next to another sequence, in a
-    # slot that was used before: state must have been reset and carried correctly
-    s1, s2 = eng.start_sequence(), eng.start_sequence()
-    other = util.random_tokens(cfg.vocab_size, 40, 4)
-    out = [eng.step([Entry(s1, other[:30]), Entry(s2, toks[:50], want=list(range(50)))]).cpu()]
-    for i in range(50, 90):
-        entries = [Entry(s2, [toks[i]], want=[0])]
-        if i < 60:
-            entries.insert(0, Entry(s1, [other[i - 20]]))
-        out.append(eng.step(entries).cpu())
-    assert rel_err(torch.cat(out), whole) < 1e-5
-    assert not torch.isnan(whole).any() and float(whole.abs().max()) > 0
-
-
 @pytest.mark.parametrize("n_seqs", [5, 24, 40])
 def test_graph_replays_equal_eager_steps_for_any_batch_size(tmp_path_factory, n_seqs):
     """The captured step is replayed many times with eager work and synchronisations in
@@ -463,3 +377,243 @@ def test_layers_with_windows_have_storage_of_their_own(tmp_path_factory, dtype, 
     eng.end_sequence(a)
     eng.end_sequence(b)
     assert all(g.pages.held == 0 for _, g in eng.cache.kv_groups)
+
+
+def test_trace_run_chunks_and_a_mixed_step(tmp_path_factory, tmp_path):
+    """bin/trace_run on steps the generation loop never makes: a request fed as chunks of 37,
+    29, 1 and 33 tokens, and one step that holds single tokens, a 40-token chunk at position
+    70 and a fresh 130-token prompt.  float32 logits are bit-equal to the whole sequences'."""
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg, w = plain.load_folder(folder)
+    V = cfg["vocab"]
+    seqs, before, mixed = util.mixed_step_case(V)
+    seqs["k"] = util.random_tokens(V, 100, 21)
+    steps, where = [], {r: [] for r in seqs}
+
+    def add(parts, end=()):
+        n = len(steps)
+        at = 0
+        entries = []
+        for r, lo, count in parts:
+            entries.append({"id": r, "tokens": seqs[r][lo:lo + count], "want": list(range(count))})
+            where[r].append((n, at, count))
+            at += count
+        steps.append({"step": n, "entries": entries, "end": list(end)})
+
+    at = 0
+    for n in (37, 29, 1, 33):
+        add([("k", at, n)], end=["k"] if at + n == 100 else [])
+        at += n
+    add([(r, 0, before[r]) for r in ("d0", "d1", "d2", "c")])
+    add([(r, before.get(r, 0), mixed[r]) for r in ("d0", "c", "d1", "p", "d2")],
+        end=["d0", "d1", "d2"])
+    add([("c", 110, 1), ("p", 130, 1)], end=["p"])
+    add([("c", 111, 1)], end=["c"])
+    most = 64 + 128 + 192 + 128 + 192           # d0, d1, d2, c, p live together, in pages
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        out = str(tmp_path / dtype)
+        _replay(folder, dtype, steps, out, most)
+        eng = engine_for(folder, dtype) if dtype == "float32" else None
+        for r, toks in seqs.items():
+            rows = []
+            for step, row, count in where[r]:
+                data = np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, V)
+                rows.append(torch.from_numpy(data[row:row + count].copy()))
+            got = torch.cat(rows)
+            assert rel_err(got, plain.forward(w, cfg, toks)) < tol, (dtype, r)
+            if eng is not None:
+                from gpt_fast_amd import Entry
+                slot = eng.start_sequence()
+                whole = eng.step([Entry(slot, toks, want=list(range(len(toks))))]).cpu()
+                eng.end_sequence(slot)
+                assert torch.equal(got, whole), r
+
+
+def test_generation_in_bfloat16_with_rows_that_retire_mid_session(tmp_path_factory):
+    """24 requests in batches of 20 and 4, bfloat16, a stop token that ends several requests
+    at different steps: the recorded step is replayed with filler rows in place of the ended
+    requests, over more than sixteen rows (the vendor library's products inside the
+    recording).  The tokens equal those of the same run without a recording."""
+    import gpt_fast_amd as gfa
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg = plain.read_config(folder)
+    prompts = [util.random_tokens(cfg["vocab"], 1 + (5 * i) % 31, 500 + i) for i in range(24)]
+    eng = engine_for(folder, "bfloat16", max_tokens=64 * 20)
+    free = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, use_graph=False).tokens
+    # a token that some requests draw early and others late or never
+    counts = {}
+    for t in free:
+        for tok in set(t[2:20]):
+            counts[tok] = counts.get(tok, 0) + 1
+    stop = max(counts, key=lambda k: (min(counts[k], 24 - counts[k]), k))
+    runs = {}
+    for use_graph in (False, True):
+        res = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=20,
+                           stop_tokens=[stop], use_graph=use_graph)
+        runs[use_graph] = res
+        assert eng.cache.slots.held == 0
+        eng.cache.check()
+    assert runs[True].tokens == runs[False].tokens
+    assert runs[True].finish_reasons == runs[False].finish_reasons
+    ended = [i for i, r in enumerate(runs[True].finish_reasons) if r == "stop"]
+    assert 2 <= len(ended) < 24
+    assert len({len(runs[True].tokens[i]) for i in ended}) > 1      # at different steps
+    for i in ended:
+        assert runs[True].tokens[i][-1] == stop and stop not in runs[True].tokens[i][:-1]
+    # sampled, with a seed: also the same with and without the recording
+    kw = dict(max_new_tokens=12, temperature=0.9, top_k=30, batch_size=20, stop_tokens=[stop])
+    a = gfa.generate(eng, prompts, seed=5, use_graph=True, **kw).tokens
+    b = gfa.generate(eng, prompts, seed=5, use_graph=False, **kw).tokens
+    c = gfa.generate(eng, prompts, seed=6, use_graph=True, **kw).tokens
+    assert a == b and a != c
+
+
+def test_the_recorded_step_is_kept_across_calls(tmp_path_factory):
+    """generate() records the one-token step once per shape and sampling law; later calls
+    of that shape replay it (the reference compiles its decode step once for all samples,
+    generate.py:338-345), also for another seed, which lives in the step's buffer."""
+    import gpt_fast_amd as gfa
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "A")
+    cfg, w = plain.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 60 + n) for n in (7, 3, 12)]
+    eng = engine_for(folder, "float32")
+    want = [plain.greedy_generate(w, cfg, p, 8) for p in prompts]
+    assert gfa.generate(eng, prompts, max_new_tokens=8, temperature=0.0).tokens == want
+    assert len(eng.recorded_steps) == 1
+    first = next(iter(eng.recorded_steps._steps.values()))
+    graph = first.graph
+    assert graph is not None and not first.busy
+    # other prompts of the same lengths: the same recording, right tokens
+    prompts2 = [util.random_tokens(cfg["vocab"], n, 80 + n) for n in (7, 3, 12)]
+    want2 = [plain.greedy_generate(w, cfg, p, 8) for p in prompts2]
+    assert gfa.generate(eng, prompts2, max_new_tokens=8, temperature=0.0).tokens == want2
+    assert len(eng.recorded_steps) == 1 and first.graph is graph
+    # sampling is another law (one more recording); seeds share it
+    kw = dict(max_new_tokens=8, temperature=0.8, top_k=50)
+    a = gfa.generate(eng, prompts, seed=1, **kw).tokens
+    b = gfa.generate(eng, prompts, seed=2, **kw).tokens
+    assert len(eng.recorded_steps) == 2
+    assert a != b
+    assert a == gfa.generate(eng, prompts, seed=1, use_graph=False, **kw).tokens
+    assert b == gfa.generate(eng, prompts, seed=2, use_graph=False, **kw).tokens
+    # two sessions of one shape open at once do not share buffers
+    from gpt_fast_amd.engine.decode import DecodeSession
+    from gpt_fast_amd.sampling import SamplingParams
+    slots = [eng.start_sequence() for _ in range(2)]
+    from gpt_fast_amd import Entry
+    eng.step([Entry(s, [1, 2, 3]) for s in slots])
+    tok = torch.tensor([4], dtype=torch.int32, device="cuda:0")
+    s1 = DecodeSession(eng, slots[:1], [0], tok, SamplingParams(temperature=0.0), max_new_tokens=4)
+    s2 = DecodeSession(eng, slots[1:], [1], tok, SamplingParams(temperature=0.0), max_new_tokens=4)
+    assert s1.rec is not s2.rec
+    t1, t2 = s1.collect(s1.launch()), s2.collect(s2.launch())
+    assert t1 == t2                                  # equal sequences, equal tokens
+    s1.close(), s2.close()
+    for s in slots:
+        eng.end_sequence(s)
+
+
+def test_generate_checks_room_before_it_runs(tmp_path_factory):
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.cache.slots import CacheFull
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")           # 128 positions
+    eng = engine_for(folder, "float32", max_tokens=64 * 3, max_sequences=3)
+    with pytest.raises(ValueError, match="128 positions"):
+        gfa.generate(eng, [[1] * 100], max_new_tokens=29, temperature=0.0)
+    with pytest.raises(CacheFull):                   # 65 + 64 + 1 tokens: four pages
+        gfa.generate(eng, [[1] * 60, [2] * 60, [3]], max_new_tokens=6, temperature=0.0)
+    with pytest.raises(CacheFull):                   # four sequences, three slots
+        gfa.generate(eng, [[1], [2], [3], [4]], max_new_tokens=2, temperature=0.0)
+    assert eng.cache.slots.held == 0
+    # the same requests in batches that fit
+    out = gfa.generate(eng, [[1], [2], [3], [4]], max_new_tokens=2, temperature=0.0, batch_size=2)
+    assert [len(t) for t in out.tokens] == [2, 2, 2, 2]
+
+
+# --------------------------------------------------------------------------------------
+# the command line, as a program (reference generate.py:272-437, 440-470)
+def _cli(*args, timeout=110):
+    proc = subprocess.run([sys.executable, "-m", "gpt_fast_amd", *map(str, args)], cwd=ROOT,
+                          capture_output=True, text=True, timeout=timeout)
+    return proc
+
+
+def test_command_line_generates_the_plain_tokens(tmp_path_factory):
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    cfg, w = plain.load_folder(folder)
+    prompt = util.random_tokens(cfg["vocab"], 9, 44)
+    want = plain.greedy_generate(w, cfg, prompt, 8)
+    proc = _cli("--checkpoint_path", folder, "--prompt_ids", ",".join(map(str, prompt)),
+                "--temperature", 0, "--num_samples", 2, "--max_new_tokens", 8, "--dtype", "float32")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.splitlines()
+    shown = [l for l in lines if l.strip() and all(p.isdigit() for p in l.split())]
+    assert len(shown) == 2                            # one line of ids per sample
+    for l in shown:
+        assert [int(t) for t in l.split()] == prompt + want
+    for needle in ("Time for inference 1:", "Time for inference 2:", "Bandwidth achieved:",
+                   "FLOPS achieved:", "Batch Size: 1", "Prompt Length: 9", "Generated tokens: 8",
+                   "Average tokens/sec:", "Memory used:"):
+        assert any(needle in l for l in lines), needle
+
+
+def test_command_line_random_weights_and_a_batch(tmp_path):
+    proc = _cli("--random", "tiny-llama-b", "--prompt", 5, "--batch_size", 3, "--num_samples", 2,
+                "--max_new_tokens", 6, "--top_k", 40)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = proc.stdout
+    assert "Only displaying the first generation of the batch" in out
+    assert "Batch Size: 3" in out and "Prompt Length: 5" in out
+    shown = [l for l in out.splitlines() if l.strip() and all(p.isdigit() for p in l.split())]
+    assert len(shown) == 2 and all(len(l.split()) == 11 for l in shown)
+    # the preset may also be a config.json file; the architecture comes from the file
+    import json as _json
+    path = tmp_path / "config.json"
+    path.write_text(_json.dumps(util.TINY_C))
+    proc = _cli("--random", path, "--prompt", 4, "--num_samples", 1, "--max_new_tokens", 3,
+                "--dtype", "float32")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "Prompt Length: 4" in proc.stdout
+
+
+def test_command_line_refusals(tmp_path_factory):
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "A")
+    for args, needle in (
+            (["--checkpoint_path", folder, "--interactive"], "interactive"),
+            (["--checkpoint_path", folder, "--speculate_k", 4], "speculative"),
+            (["--prompt", 4], "either --checkpoint_path"),
+            (["--checkpoint_path", folder, "--random", "7B"], "either --checkpoint_path"),
+            (["--checkpoint_path", folder, "--prompt", "some text"], "tokenizer"),
+            (["--random", "no-such-model", "--prompt", 4], "preset"),
+            (["--checkpoint_path", folder, "--prompt", 60, "--max_new_tokens", 10,
+              "--num_samples", 1], "64 positions")):
+        proc = _cli(*args)
+        assert proc.returncode != 0, args
+        assert needle in (proc.stderr + proc.stdout), (args, proc.stderr[-500:])
+
+
+def test_command_line_text_prompt_starts_with_bos(tmp_path_factory, tmp_path):
+    """A folder with only a tokenizer.json (the Llama-3 family's kind): the text prompt is
+    encoded with the BOS id of config.json in front (generate.py:213-217)."""
+    import json as _json
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    src = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(src, folder)
+    cfg_path = os.path.join(folder, "config.json")
+    c = _json.load(open(cfg_path))
+    c["bos_token_id"] = 7
+    _json.dump(c, open(cfg_path, "w"))
+    vocab = {f"w{i}": i for i in range(c["vocab_size"])}
+    tk = Tokenizer(models.WordLevel(vocab, unk_token="w0"))
+    tk.pre_tokenizer = pre_tokenizers.Whitespace()
+    tk.save(os.path.join(folder, "tokenizer.json"))
+    pcfg, w = plain.load_folder(folder)
+    want = plain.greedy_generate(w, pcfg, [7, 21, 5, 300], 5)
+    proc = _cli("--checkpoint_path", folder, "--prompt", "w21 w5 w300", "--temperature", 0,
+                "--num_samples", 1, "--max_new_tokens", 5, "--dtype", "float32")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "Prompt Length: 4" in proc.stdout
+    text = " ".join(f"w{t}" for t in [7, 21, 5, 300] + want)
+    assert text in proc.stdout

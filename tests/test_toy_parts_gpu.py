@@ -252,3 +252,224 @@ def test_run_order_is_data_a_layer_twice_and_a_borrowed_cache():
     x = _plain_dense_ffn(x, w, "layers.0.", pcfg)
     want = plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
     _steps_equal_whole(eng, toks, want, cfg.vocab_size, TOL_F32)
+
+
+# --------------------------------------------------------------------------------------
+# A mixer with fixed-size state of its own (no keys or values): a running mean of its
+# inputs; state per sequence = [sum of inputs, count].  Two forms: one loops over the
+# batch on the host (so its steps cannot be recorded), one works from the batch's device
+# fields alone and says ``replayable``.
+@dataclasses.dataclass(frozen=True)
+class RunningMeanSpec:
+    dim: int
+    kind: str = "toy_running_mean"
+
+
+def _running_mean_classes():
+    from gpt_fast_amd.cache.store import StateNeed
+    from gpt_fast_amd.parts import Param, Part
+
+    class RunningMean(Part):
+        def __init__(self, spec, rt):
+            self.spec, self.rt = spec, rt
+
+        def parameters(self):
+            return {"mix": Param((self.spec.dim, self.spec.dim))}
+
+        def bind(self, tensors):
+            self.mix = tensors["mix"]
+
+        def cache_need(self):
+            return StateNeed((self.spec.dim + 1,), "float32")
+
+        def forward(self, x, batch, entry, residual):
+            state = entry.state                                   # [n_slots + 1, dim + 1]
+            q_start = batch.host_field("q_start")
+            slots = batch.host_field("slots")
+            for b in range(batch.n_seqs):
+                lo, hi = int(q_start[b]), int(q_start[b + 1])
+                xs = x[lo:hi].float()
+                s = state[int(slots[b])]
+                sums = s[:-1] + torch.cumsum(xs, 0)
+                counts = s[-1] + torch.arange(1, hi - lo + 1, device=x.device)
+                residual[lo:hi] += (sums / counts[:, None]) @ self.mix.float().T
+                s[:-1] = sums[-1]
+                s[-1] = counts[-1]
+
+    class RunningMeanOnDevice(RunningMean):
+        """The same from device fields only: the same kernels whatever the batch holds."""
+        replayable = True
+
+        def forward(self, x, batch, entry, residual):
+            state = entry.state
+            n = x.shape[0]
+            seq = batch.tok_seq.long()
+            slot = batch.slots.long()[seq]                        # of every token
+            idx = torch.arange(n, device=x.device)
+            earlier = ((seq[:, None] == seq[None, :]) & (idx[:, None] >= idx[None, :])).float()
+            old = state[slot]
+            sums = earlier @ x.float() + old[:, :-1]
+            counts = (earlier @ torch.ones(n, 1, device=x.device))[:, 0] + old[:, -1]
+            residual += (sums / counts[:, None]) @ self.mix.float().T
+            last = batch.q_start[1:].long() - 1                   # each sequence's last token
+            state[batch.slots.long()] = torch.cat([sums[last], counts[last, None]], 1)
+
+    return RunningMean, RunningMeanOnDevice
+
+
+def _toy_state_model(on_device: bool):
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.config.spec import LayerSpec, ModelPlan, NormSpec, Run
+    from gpt_fast_amd.parts import Runtime, register_mixer
+    from gpt_fast_amd.parts.model import DecoderModel
+    host_form, device_form = _running_mean_classes()
+    register_mixer("toy_running_mean", device_form if on_device else host_form)
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_A)
+    base = arch.plan(cfg)
+    D = cfg.hidden_size
+    toy_layer = LayerSpec(name="toy", mixer=RunningMeanSpec(D), mixer_norm=NormSpec(D, 1e-5),
+                          feed_forward=base.layers[0].feed_forward,
+                          feed_forward_norm=NormSpec(D, 1e-5))
+    # attention, toy, attention, toy again (a state entry of its own), then the first layer
+    # again with the first run's keys and values (borrowed)
+    plan = ModelPlan(dim=D, vocab_size=cfg.vocab_size,
+                     layers=[base.layers[0], toy_layer, base.layers[1]],
+                     order=[Run(0), Run(1), Run(2), Run(1), Run(0, cache_from=0)],
+                     final_norm=base.final_norm, max_positions=4096)
+    model = DecoderModel(plan, Runtime(torch.float32, DEV))
+    w = _random_parameters(model, 31)
+    eng = gfa.Engine.from_plan(plan, {k: v.to(DEV) for k, v in w.items()}, "float32", DEV,
+                               max_tokens=1024, max_sequences=6)
+    return eng, w, plain.config_from_dict(util.TINY_A), cfg.vocab_size
+
+
+def _plain_toy_state_logits(w, pcfg, toks):
+    """The toy plan from whole sequences with the plain parts; the running mean is
+    cumsum / count of the normed rows."""
+    def toy_block(x):
+        xn = plain.rms_norm(x, w["toy.mixer_norm.weight"], 1e-5)
+        mean = torch.cumsum(xn, 0) / torch.arange(1, x.shape[0] + 1)[:, None]
+        x = x + mean @ w["toy.mixer.mix"].T
+        hn = plain.rms_norm(x, w["toy.feed_forward_norm.weight"], 1e-5)
+        w13 = w["toy.feed_forward.w13"]
+        I = w13.shape[0] // 2
+        return x + plain.feed_forward(hn, w13[:I], w13[I:], w["toy.feed_forward.w2"])
+
+    x0 = w["tok_embeddings.weight"][torch.tensor(toks)]
+    x = _plain_dense_ffn(_plain_attention_block(x0, w, "layers.0.", pcfg), w, "layers.0.", pcfg)
+    x = toy_block(x)
+    x = _plain_dense_ffn(_plain_attention_block(x, w, "layers.1.", pcfg), w, "layers.1.", pcfg)
+    x = toy_block(x)
+    x = _plain_dense_ffn(_plain_attention_block(x, w, "layers.0.", pcfg, kv_of=x0), w, "layers.0.", pcfg)
+    return plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_toy_mixer_with_state_registers_and_steps(on_device):
+    """A mixer defined here, with fixed-size state per sequence and no keys or values, is
+    registered, built into a plan next to attention layers, and stepped: no file of the
+    library changes.  Compared with the plain computation over the whole sequence: whole,
+    cut into steps beside another sequence, in slots that were used before."""
+    eng, w, pcfg, V = _toy_state_model(on_device)
+    assert len(eng.cache.groups) == 2             # one KV group, one state group of two entries
+    assert eng.model.replayable == on_device
+    toks = util.random_tokens(V, 90, 3)
+    want = _plain_toy_state_logits(w, pcfg, toks)
+    _steps_equal_whole(eng, toks, want, V, TOL_F32)
+    _steps_equal_whole(eng, toks, want, V, TOL_F32)          # again: slots and state reused
+    assert eng.cache.slots.held == 0
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_toy_mixer_with_state_through_generate(on_device):
+    """The same model through generate(): the decode session warms up before it records,
+    which must not count a token twice into the state; rows that end at a stop token stay
+    as fillers and must not write another sequence's state; the host-looping form is
+    stepped without a recording although one is asked for.  Every token must be the best
+    by the plain logits of the request's own sequence."""
+    import gpt_fast_amd as gfa
+    eng, w, pcfg, V = _toy_state_model(on_device)
+    prompts = [util.random_tokens(V, n, 400 + n) for n in (5, 1, 17, 9)]
+    free = gfa.generate(eng, prompts, max_new_tokens=14, temperature=0.0, use_graph=False).tokens
+    stop = free[2][5]                              # request 2 ends after six tokens at the latest
+    runs = {}
+    for use_graph in (False, True):
+        for _ in range(2):                         # the second time the recording is replayed
+            res = gfa.generate(eng, prompts, max_new_tokens=14, temperature=0.0,
+                               stop_tokens=[stop], use_graph=use_graph)
+        runs[use_graph] = res.tokens
+        assert eng.cache.slots.held == 0
+    assert runs[True] == runs[False]
+    assert len(runs[True][2]) <= 6 and runs[True][2][-1] == stop
+    assert len(eng.recorded_steps) >= 1
+    recorded = [s.graph is not None for s in eng.recorded_steps._steps.values()]
+    assert any(recorded) == on_device
+    for p, new in zip(prompts, runs[True]):
+        logits = _plain_toy_state_logits(w, pcfg, p + new)
+        for i, tok in enumerate(new):
+            row = logits[len(p) - 1 + i]
+            assert float(row[tok]) >= float(row.max()) - 1e-4 * float(row.abs().max()), (i, tok)
+
+
+def test_plan_level_steps_scale_position_and_cap():
+    """What a plan may state around its layers, none of which Llama uses: a factor on the
+    embedded rows, a position encoding added to them (a toy table of learned vectors,
+    registered here), a factor and a soft cap on the logits."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.parts import Param, Part, register_position
+    from gpt_fast_amd.parts import Runtime
+    from gpt_fast_amd.parts.model import DecoderModel
+
+    @dataclasses.dataclass(frozen=True)
+    class LearnedTableSpec:
+        dim: int
+        positions: int
+        kind: str = "toy_learned_table"
+
+    class LearnedTable(Part):
+        replayable = True
+
+        def __init__(self, spec, rt):
+            self.spec = spec
+
+        def parameters(self):
+            return {"table": Param((self.spec.positions, self.spec.dim))}
+
+        def bind(self, tensors):
+            self.table = tensors["table"]
+
+        def add_to_stream(self, residual, batch):
+            residual += self.table.float()[batch.tok_pos.long()]
+
+    register_position("toy_learned_table", LearnedTable)
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_B)
+    plan = arch.plan(cfg)
+    plan.embedding_scale = 1.7
+    plan.input_position = LearnedTableSpec(cfg.hidden_size, 200)
+    plan.logit_scale = 3.0
+    plan.logit_softcap = 2.5
+    model = DecoderModel(plan, Runtime(torch.float32, DEV))
+    w = _random_parameters(model, 41)
+    assert "input_position.table" in w
+    eng = gfa.Engine.from_plan(plan, {k: v.to(DEV) for k, v in w.items()}, "float32", DEV,
+                               max_tokens=1024)
+    pcfg = plain.config_from_dict(util.TINY_B)
+    toks = util.random_tokens(cfg.vocab_size, 100, 12)
+    x = w["tok_embeddings.weight"][torch.tensor(toks)] * 1.7 + w["input_position.table"][:100]
+    for i in range(cfg.num_hidden_layers):
+        x = _plain_dense_ffn(_plain_attention_block(x, w, f"layers.{i}.", pcfg), w, f"layers.{i}.", pcfg)
+    logits = plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
+    want = 2.5 * torch.tanh(logits * 3.0 / 2.5)
+    _steps_equal_whole(eng, toks, want, cfg.vocab_size, TOL_F32)
+    # greedy generation through the recorded step agrees with stepping
+    a = gfa.generate(eng, [toks[:10], toks[:3]], max_new_tokens=6, temperature=0.0).tokens
+    b = gfa.generate(eng, [toks[:10], toks[:3]], max_new_tokens=6, temperature=0.0,
+                     use_graph=False).tokens
+    assert a == b
+    # a position part without add_to_stream cannot stand there
+    plan2 = arch.plan(cfg)
+    plan2.input_position = plan2.layers[0].mixer.position
+    with pytest.raises(TypeError, match="add_to_stream"):
+        DecoderModel(plan2, Runtime(torch.float32, DEV))

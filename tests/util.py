@@ -76,3 +76,14 @@ def rel_err(a, b):
 # also rounds activations to bfloat16 between kernels.
 TOL_F32 = 2e-5
 TOL_BF16 = 4e-2
+
+
+def mixed_step_case(V):
+    """Five sequences; one step brings three of them one token each, one a chunk of 40
+    tokens at position 70, one a fresh prompt of 130 tokens."""
+    seqs = {"d0": random_tokens(V, 9, 31), "d1": random_tokens(V, 66, 32),
+            "d2": random_tokens(V, 130, 33), "c": random_tokens(V, 112, 34),
+            "p": random_tokens(V, 131, 35)}
+    before = {"d0": 8, "d1": 65, "d2": 129, "c": 70}            # fed by the earlier step
+    mixed = {"d0": 1, "d1": 1, "d2": 1, "c": 40, "p": 130}      # fed by the mixed step
+    return seqs, before, mixed

@@ -7,11 +7,19 @@ A step is one decode step of a batch of 8 sequences (128-token random prompts, c
 W untimed steps, then exactly K timed steps between device synchronisations.  Prints one
 JSON line: ``value`` is decoded tokens per second; ``prefill`` is one 2,048-token prompt;
 ``roofline`` compares the bytes a decode step must read (every weight once, the cache of
-the live sequences) per second with the HBM peak; ``points`` holds decode at batch 1 and 64.
+the live sequences) per second with the HBM peak; ``points`` holds decode at batch 1 and 64;
+``vs_baseline`` compares the batch-1 point with the reference's published batch-1 number.
+
+Other workloads of the same program: ``--preset`` (another shape), ``--context`` (cache
+positions per sequence), ``--prompt-lens LO:HI`` (prompts of unequal, seeded random lengths;
+adds the ragged prefill's tokens per second), ``--prefill-only`` (just the timed prompt, for
+profiling), ``--ceilings`` (what this GPU reaches with a bare read stream and a bare
+matrix-instruction loop, beside the datasheet peaks).
 """
 import argparse
 import json
 import os
+import random
 import sys
 import time
 
@@ -27,25 +35,31 @@ def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def decode_run(engine, batch, prompt_len, warmup, steps, use_graph=True):
-    """(seconds per step, bytes a step reads) for `steps` decode steps of `batch` sequences."""
+def decode_run(engine, prompt_lens, warmup, steps, use_graph=True):
+    """(seconds per step, bytes a step reads, seconds of the prefill) for ``steps`` decode
+    steps of sequences with the given prompt lengths."""
     import torch
     from gpt_fast_amd import Entry
     from gpt_fast_amd.engine.decode import DecodeSession
     from gpt_fast_amd.sampling import SamplingParams, sample
+    batch = len(prompt_lens)
     g = torch.Generator().manual_seed(batch)
     V = engine.vocab_size
     slots = [engine.start_sequence() for _ in range(batch)]
-    entries = [Entry(s, torch.randint(0, V, (prompt_len,), generator=g).tolist(),
-                     want=[prompt_len - 1], key=i) for i, s in enumerate(slots)]
+    entries = [Entry(s, torch.randint(0, V, (n,), generator=g).tolist(), want=[n - 1], key=i)
+               for i, (s, n) in enumerate(zip(slots, prompt_lens))]
     params = SamplingParams(temperature=0.0)
     # prefill in pieces of at most 8 prompts to bound activation memory
     first = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
     for i in range(0, batch, 8):
         b = engine.prepare(entries[i:i + 8])
         logits = engine.model.forward(b, engine.cache)
         first.append(sample(logits, params, b.row_keys, None))
     first = torch.cat(first)
+    torch.cuda.synchronize()
+    prefill_seconds = time.perf_counter() - t0
     sess = DecodeSession(engine, slots, list(range(batch)), first, params, use_graph=use_graph,
                          max_new_tokens=warmup + steps + 1)
     for _ in range(warmup):
@@ -56,13 +70,14 @@ def decode_run(engine, batch, prompt_len, warmup, steps, use_graph=True):
         sess.advance()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+    sess.close()
     # bytes of the middle step: weights once + keys and values of every live token
-    ctx = prompt_len + warmup + steps // 2
-    kv_bytes = sum(g.bytes_per_token() for _, g in engine.cache.kv_groups) * ctx * batch
+    ctx = sum(n + warmup + steps // 2 for n in prompt_lens)
+    kv_bytes = sum(g.bytes_per_token() for _, g in engine.cache.kv_groups) * ctx
     step_bytes = engine.model.parameter_bytes() + kv_bytes
     for s in slots:
         engine.end_sequence(s)
-    return dt, step_bytes
+    return dt, step_bytes, prefill_seconds
 
 
 def prefill_run(engine, n_tokens, repeats=3):
@@ -103,8 +118,15 @@ def main():
     ap.add_argument("--batch", type=int, default=8, help="sequences decoded together (headline: 8)")
     ap.add_argument("--preset", default="llama-3.1-8b",
                     help="shape to run (headline: llama-3.1-8b; others: 7B, llama-3.1-70b, ...)")
+    ap.add_argument("--architecture", default=None, help="architecture that knows the preset")
     ap.add_argument("--prompt-len", type=int, default=128)
+    ap.add_argument("--prompt-lens", default=None, metavar="LO:HI",
+                    help="prompts of unequal lengths, uniform in [LO, HI], seeded")
+    ap.add_argument("--context", type=int, default=4096, help="cache positions per sequence")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the timed prompt")
+    ap.add_argument("--prefill-only", action="store_true", help="time the prompt and nothing else")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="also measure a bare read stream, a copy and a matrix-instruction loop")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
     args = ap.parse_args()
@@ -114,18 +136,25 @@ def main():
 
     import torch
     import gpt_fast_amd as gfa
-    from gpt_fast_amd.config.llama import LlamaConfig, preset_dict
 
-    raw = preset_dict(args.preset)
+    arch, cfg = gfa.find_preset(args.preset, args.architecture)
+    raw = arch.config_dict(cfg)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
-    cfg = LlamaConfig.from_dict(raw)
-    batch, context, prompt_len = args.batch, 4096, args.prompt_len
+        cfg = arch.read_config(raw)
+    batch, context = args.batch, args.context
+    if args.prompt_lens:
+        lo, hi = (int(v) for v in args.prompt_lens.split(":"))
+        rng = random.Random(batch)
+        prompt_lens = [rng.randint(lo, hi) for _ in range(batch)]
+    else:
+        prompt_lens = [args.prompt_len] * batch
+    rows = batch if args.no_points or args.prefill_only else max(64, batch)
     t0 = time.time()
-    engine = gfa.Engine.from_random("llama", cfg, seed=0, dtype="bfloat16", device="cuda:0",
-                                    max_tokens=max(64, batch) * context,
-                                    max_sequences=max(64, batch))
+    engine = gfa.Engine.from_random(arch.names[0], cfg, seed=0, dtype="bfloat16", device="cuda:0",
+                                    max_tokens=max(rows * context, args.prefill_tokens + 64),
+                                    max_sequences=rows)
     torch.cuda.synchronize()
     log(f"[bench] model ready in {time.time() - t0:.1f} s")
 
@@ -138,14 +167,32 @@ def main():
          ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
          if k in rs])
     use_graph = not args.no_graph
-    dt, step_bytes = decode_run(engine, batch, prompt_len, args.warmup, args.steps, use_graph)
+    T = args.prefill_tokens
+
+    def prefill_point():
+        pt = prefill_run(engine, T)
+        flops = prefill_flops(cfg, cfg.num_hidden_layers, T)
+        log(f"[bench] prefill {T}: {pt * 1e3:.2f} ms")
+        return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                "frac": round(flops / pt / 1e12 / MFMA_PEAK_TFLOPS["bf16"], 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"metric": f"prefill tok/s @ {T} tokens; {model_name} bf16",
+                          "n_layer": cfg.num_hidden_layers, "prefill": prefill_point()}), flush=True)
+        return
+
+    if max(prompt_lens) + args.warmup + args.steps + 1 > context:
+        print(f"prompt ({max(prompt_lens)}) + {args.warmup + args.steps + 1} decoded tokens exceed "
+              f"--context {context}")
+        sys.exit(2)
+    dt, step_bytes, prefill_s = decode_run(engine, prompt_lens, args.warmup, args.steps, use_graph)
     value = batch / dt
     log(f"[bench] decode b{batch}: {dt * 1e3:.3f} ms/step, {value:.1f} tok/s")
     out = {
         "metric": f"decode tok/s @ batch {batch}; {model_name} bf16", "value": round(value, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": round(value / BASELINE_TOK_S, 3) if headline else None,
+        "vs_baseline": round(value / BASELINE_TOK_S, 3) if headline and batch == 1 else None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
             "model": args.preset, "n_layer": cfg.num_hidden_layers,
@@ -155,7 +202,8 @@ def main():
             "vocab_size": cfg.vocab_size, "rope_base": cfg.rope_theta,
             "rope_scaling": scaling,
             "norm_eps": cfg.rms_norm_eps, "global_batch": batch, "seq_len": context,
-            "prompt_len": prompt_len, "new_tokens": args.warmup + args.steps,
+            "prompt_len": args.prompt_lens or args.prompt_len,
+            "new_tokens": args.warmup + args.steps,
             "weights": "random N(0,0.02) bf16", "sampling": "greedy", "hip_graph": use_graph,
             "parallelism": "single GPU",
         },
@@ -163,20 +211,30 @@ def main():
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)},
     }
+    if args.prompt_lens:
+        # the unequal prompts went through the engine in one step per eight of them
+        out["ragged_prefill"] = {"value": round(sum(prompt_lens) / prefill_s, 1),
+                                 "tokens": sum(prompt_lens), "ms": round(prefill_s * 1e3, 3),
+                                 "lengths": " ".join(map(str, prompt_lens))}
     if not args.no_points:
-        T = args.prefill_tokens
-        pt = prefill_run(engine, T)
-        flops = prefill_flops(cfg, cfg.num_hidden_layers, T)
-        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                          "frac": round(flops / pt / 1e12 / MFMA_PEAK_TFLOPS["bf16"], 4)}
-        log(f"[bench] prefill {T}: {pt * 1e3:.2f} ms")
+        out["prefill"] = prefill_point()
         points = {}
         for b in (1, 64):
             steps = min(args.steps, 128)
-            d, _ = decode_run(engine, b, prompt_len, min(args.warmup, 8), steps, use_graph)
+            d, _, _ = decode_run(engine, [args.prompt_len] * b, min(args.warmup, 8), steps, use_graph)
             points[f"decode_b{b}"] = round(b / d, 2)
             log(f"[bench] decode b{b}: {d * 1e3:.3f} ms/step, {b / d:.1f} tok/s")
         out["points"] = points
+        if headline:
+            # like for like: the reference's published number is its batch-1 decode speed
+            out["vs_baseline"] = round(points["decode_b1"] / BASELINE_TOK_S, 3)
+            out["vs_baseline_point"] = "decode_b1"
+    if args.ceilings:
+        from gpt_fast_amd.ops import ceilings
+        c = ceilings.measure("cuda:0")
+        c["decode_frac_of_read_stream"] = round(step_bytes / dt / 1e9 / c["hbm_read_gbs"], 4)
+        out["ceilings"] = c
+        log(f"[bench] ceilings: {c}")
     print(json.dumps(out), flush=True)
 
 

@@ -103,9 +103,11 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) {
+                // every lane loads (dims beyond the head: the row's first chunk), then those
+                // lanes are cleared: no load runs under a partial execution mask
                 const int d = ds * 32 + lg * 8;
-                kf[kt][ds].u = (d < hd) ? *(const uint4*)(kbase + (size_t)(8 * (li >> 2) + 4 * kt + (li & 3)) * hd + d)
-                                        : make_uint4(0, 0, 0, 0);
+                const uint4 got = *(const uint4*)(kbase + (size_t)(8 * (li >> 2) + 4 * kt + (li & 3)) * hd + (d < hd ? d : 0));
+                kf[kt][ds].u = (d < hd) ? got : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -177,11 +179,13 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
             // the running maximum rarely moves after the first blocks: skip the rescale then
             const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
 #pragma unroll
+            // every tile of dims is multiplied, also those beyond the head (their values are
+            // zero and never stored): with a branch on the head size between the matrix
+            // instructions, the two-tile kernel with prefetch gave wrong sums for its first
+            // tile at head size 16 once a second block of keys was read
             for (int dt = 0; dt < DT; ++dt) {
-                if (dt * 16 < hd) {
-                    if (rescale) o[rt][dt] *= alpha;
-                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
-                }
+                if (rescale) o[rt][dt] *= alpha;
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
             }
         }
     };
@@ -524,16 +528,17 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         }
         __builtin_amdgcn_s_setprio(1);
 #pragma unroll
+        // every tile of dims is multiplied, also those beyond a smaller head (what LDS holds
+        // there goes into accumulators that are never stored): a branch between matrix
+        // instructions on the same accumulators has given wrong sums
         for (int dt = 0; dt < DT; ++dt) {
-            if (FULL || dt * 16 < hd) {
 #pragma unroll
-                for (int hb = 0; hb < 2; ++hb) {
-                    Frag vf;
-                    vf.u = *(const uint4*)(vt + dt * 16 * VROW + v_off[hb]);
+            for (int hb = 0; hb < 2; ++hb) {
+                Frag vf;
+                vf.u = *(const uint4*)(vt + dt * 16 * VROW + v_off[hb]);
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt)
-                        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
-                }
+                for (int rt = 0; rt < RT; ++rt)
+                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
             }
         }
         __builtin_amdgcn_s_setprio(0);

@@ -439,7 +439,8 @@ def test_generation_in_bfloat16_with_rows_that_retire_mid_session(tmp_path_facto
     cfg = plain.read_config(folder)
     prompts = [util.random_tokens(cfg["vocab"], 1 + (5 * i) % 31, 500 + i) for i in range(24)]
     eng = engine_for(folder, "bfloat16", max_tokens=64 * 20)
-    free = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, use_graph=False).tokens
+    free = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=20,
+                        use_graph=False).tokens
     # a token that some requests draw early and others late or never
     counts = {}
     for t in free:

@@ -262,6 +262,38 @@ def _attention_over_pages(A, dtype, tol, H, G, hd, window):
         close(plain[n], ref, tol)
 
 
+@pytest.mark.parametrize("H,G,hd", [(4, 4, 16), (2, 2, 16), (6, 2, 32), (4, 4, 64), (8, 2, 128),
+                                    (4, 2, 16), (3, 1, 48), (5, 5, 80), (4, 2, 256)])
+def test_attention_of_a_chunk_at_an_offset(H, G, hd):
+    """Several new tokens of a sequence whose first tokens are cached already (start
+    position > 0), in row counts that take each form of the wave-level kernel (one, two and
+    four row tiles per wave) and the workgroup-tiled one, over one and over several blocks
+    of keys; pages beyond the newest key are poisoned."""
+    from gpt_fast_amd.ops import attention as A
+    scale = 1.0 / math.sqrt(hd)
+    for spos, qlen in [(20, 20), (13, 20), (12, 20), (37, 29), (70, 5), (33, 17), (67, 33),
+                       (100, 3), (1, 63), (130, 70)]:
+        S = spos + qlen
+        k_pages, v_pages, table, ks, vs = _paged([S], G, hd, torch.bfloat16, seed=spos + qlen)
+        g = torch.Generator().manual_seed(5)
+        q = torch.randn(qlen, H, hd, generator=g).to(torch.bfloat16)
+
+        class B:
+            pass
+        batch = B()
+        batch.tok_seq = torch.zeros(qlen, dtype=torch.int32, device=DEV)
+        batch.tok_pos = torch.arange(spos, S, dtype=torch.int32, device=DEV)
+        batch.n_tokens, batch.n_seqs = qlen, 1
+        batch.max_q_len, batch.max_kv_len, batch.is_decode = qlen, S, False
+        batch.q_start = torch.tensor([0, qlen], dtype=torch.int32, device=DEV)
+        batch.start_pos = torch.tensor([spos], dtype=torch.int32, device=DEV)
+        out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, scale, 0).cpu()
+        assert not torch.isnan(out).any(), (spos, qlen)
+        for n in range(qlen):
+            ref = _attention_ref(q[n].float(), ks[0].float(), vs[0].float(), spos + n, scale, 0)
+            close(out[n], ref, 1.5e-2)
+
+
 def test_attention_finds_one_far_key():
     """One key among hundreds stands out (its score is scaled up): the output must be
     that key's value, wherever in the cache it lies - first row, a page edge, the last."""
@@ -514,8 +546,9 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
     got = G.skinny_after_chain(xg, ssq, eps, w, out_dtype=torch.float32).double().cpu()
     for m in range(M):
         assert float((got[m] - ref[m].cpu()).abs().max() / ref[m].abs().max()) < 1.5e-2
-    from gpt_fast_amd.ops.linear import HalfNormed
-    close(HalfNormed(xg, ssq, eps).materialize(), n, 1e-2)
+    # the two halves put together by hand are the norm's rows
+    rs = torch.rsqrt(ssq.sum(0)[:M, None].double() / D + eps)
+    close(xg.double() * rs, n, 1e-2)
 
 
 @pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])

@@ -2,7 +2,7 @@
 
 Each ``<name>.hip`` becomes ``build/libgfa_<name>.so`` (plain ``hipcc -shared``, C entry
 points, no Python headers) with a stamp file beside it that holds a hash of what it was
-built from (the source, ``common.h``, the flags).  ``ensure(names)`` compiles the libraries
+built from (the source, the headers of this folder, the flags).  ``ensure(names)`` compiles the libraries
 that are asked for and are missing or whose stamp no longer fits the sources, so an edited
 kernel is never run from an old library; ``build_all()`` compiles every one anew.  Nothing
 here needs a GPU: hipcc cross-compiles.
@@ -52,7 +52,8 @@ def _build_dir() -> str:
 def source_hash(name: str) -> str:
     """Hash of everything the library of module ``name`` is built from."""
     h = hashlib.sha256()
-    for path in (os.path.join(HERE, name + ".hip"), os.path.join(HERE, "common.h")):
+    headers = sorted(f for f in os.listdir(HERE) if f.endswith(".h"))
+    for path in [os.path.join(HERE, name + ".hip")] + [os.path.join(HERE, h) for h in headers]:
         with open(path, "rb") as f:
             h.update(f.read())
         h.update(b"\0")

@@ -7,6 +7,9 @@
 //          counter-based function of (seed, row key, position, i), so a row's draw does
 //          not depend on the other rows of the launch.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
+#include <stdio.h>
 
 #define SMP_THREADS 1024
 
@@ -436,4 +439,80 @@ extern "C" int gfa_sample_split(const float* logits, size_t row_stride, int n_ro
     if (V <= 0 || !workspace) return (int)hipErrorInvalidValue;
     return run_sample_split(logits, row_stride, n_rows, V, temperature, top_k, seed, seed_dev,
                             row_keys, positions, position_offset, out, probs_out, workspace, stream);
+}
+
+// --------------------------------------------------------------------------------------
+// The same without a workspace from the caller (declared and described in sampling.h).
+// `scratch` is this library's copy of the array on each GPU; in host code its name is only
+// a handle for hipGetSymbolAddress, never an address to pass on.
+static __device__ __align__(256) unsigned char scratch[GFA_SAMPLE_STATIC_BYTES];
+
+#define GFA_MAX_DEVICES 64
+static void* scratch_of_device[GFA_MAX_DEVICES];          // the array's address on each GPU
+static std::mutex scratch_lock;
+static thread_local char last_error[256];
+
+extern "C" const char* gfa_sampling_last_error(void) { return last_error; }
+
+// The current GPU's array, looked up once per GPU with that GPU current.
+static int scratch_here(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= GFA_MAX_DEVICES) {
+        snprintf(last_error, sizeof last_error, "device %d: this library keeps scratch for devices 0..%d",
+                 dev, GFA_MAX_DEVICES - 1);
+        return (int)hipErrorInvalidDevice;
+    }
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            snprintf(last_error, sizeof last_error, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                     hipGetErrorString(e));
+            return e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+        }
+        scratch_of_device[dev] = p;
+    }
+    *out = scratch_of_device[dev];
+    return 0;
+}
+
+extern "C" int gfa_sampling_init(void) {
+    void* p = nullptr;
+    return scratch_here(&p);
+}
+
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t* __restrict__ p, size_t n) {
+    for (size_t i = blockIdx.x * (size_t)256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0;
+}
+
+extern "C" int gfa_sample_split_static(const float* logits, size_t row_stride, int n_rows, int V,
+                                       float temperature, int top_k, uint64_t seed,
+                                       const uint32_t* seed_dev, const int* row_keys,
+                                       const int* positions, int position_offset, int* out,
+                                       float* probs_out, hipStream_t stream) {
+    last_error[0] = 0;
+    if (n_rows <= 0) return 0;
+    if (V <= 0 || n_rows > GFA_SAMPLE_STATIC_MAX_ROWS || V > GFA_SAMPLE_STATIC_MAX_VOCAB ||
+        gfa_sample_split_workspace(n_rows, V) > (size_t)GFA_SAMPLE_STATIC_BYTES) {
+        snprintf(last_error, sizeof last_error,
+                 "gfa_sample_split_static: %d rows of %d logits; its fixed scratch (%d bytes per GPU) "
+                 "takes at most %d rows of at most %d logits", n_rows, V, (int)GFA_SAMPLE_STATIC_BYTES,
+                 GFA_SAMPLE_STATIC_MAX_ROWS, GFA_SAMPLE_STATIC_MAX_VOCAB);
+        return (int)hipErrorInvalidValue;
+    }
+    void* ws = nullptr;
+    const int rc = scratch_here(&ws);
+    if (rc != 0) return rc;
+    const bool histograms = temperature > 0.f && top_k > 0 && top_k < V;
+    if (histograms) {
+        // whatever the last call left where this call's histograms lie (its own layout
+        // depended on its sizes) goes; a kernel, not a memset, so that a recording replays it
+        const size_t words = (size_t)n_rows * 4 * 256;
+        clear_words_kernel<<<(unsigned)((words + 255) / 256), 256, 0, stream>>>((uint32_t*)ws, words);
+    }
+    return run_sample_split(logits, row_stride, n_rows, V, temperature, top_k, seed, seed_dev,
+                            row_keys, positions, position_offset, out, probs_out, ws, stream);
 }

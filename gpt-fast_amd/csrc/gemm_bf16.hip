@@ -240,7 +240,7 @@ struct SkinnyExtra {
     int table_stride, H, Hkv, hd, rot;
     // A norm spread over two kernels (one tile of rows).  The kernel that completes the
     // residual stream (MODE 2) also writes xg_out [M, N] = bfloat16(new residual * next_g) and
-    // ssq_out [tiles, share_rows]: each workgroup's share of its rows' sums of squares (float,
+    // ssq_out [tiles, share_rows] (tiles of gfa_skinny_tile_rows(2, N) columns): each workgroup's share of its rows' sums of squares (float,
     // from the float residual).  The next product takes xg as its x, adds the shares in a fixed
     // order (ssq_in [t_in, share_rows]) and scales its result by rsqrt(sum / K + eps): a factor per row
     // commutes with the product, so this is the RMS norm of model.py:236-241.
@@ -259,11 +259,13 @@ extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 template <int CT, int MODE, int XP = 1, bool XF = false>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
-        int N, int K, int ldo, int gate_rows, SkinnyExtra ex) {
+        int N, int K, int ldo, int gate_rows, int th, SkinnyExtra ex) {
     constexpr int RT = (MODE == 3) ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
-    const int n0 = blockIdx.x * 16;
+    // th (8..16) rows of W per workgroup: the host picks it so that the tiles divide evenly
+    // over the compute units; operand rows th..15 repeat row th - 1 and are never stored
+    const int n0 = blockIdx.x * th;
     char* stage = smem + (size_t)wave * (RT * SM_TILE);
     const int lrow = lane >> 4, lchunk = lane & 15;      // loading: row lrow + 4 j, 16-byte chunk
     const int fi = lane & 15, fg = lane >> 4;            // multiplying: row / column fi, k group fg
@@ -284,7 +286,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            int n = n0 + lrow + 4 * j;
+            const int r = lrow + 4 * j;
+            int n = n0 + (r < th ? r : th - 1);
             if (n >= N) n = N - 1;                       // clamped rows are computed, not stored
             wsrc[rt][j] = w + (size_t)(n + rt * gate_rows) * K + lchunk * 8;
         }
@@ -404,14 +407,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         res_ok[ct] = false;
         if (MODE == 2 && wave == 0) {
             const int m = ct * 16 + fi, n = n0 + fg * 4;
-            res_ok[ct] = m < M && n + 3 < N && (ldo & 3) == 0;
+            res_ok[ct] = m < M && n + 3 < N && (ldo & 3) == 0 && fg * 4 + 3 < th;
             if (res_ok[ct]) {
                 res_pre[ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
                 if (ex.xg_out) g_pre[ct] = *(const float4*)(ex.next_g + n);
             }
         }
     }
-    if (ROT_EARLY && wave == 0 && fi < M && n0 + fg * 4 < N) {
+    if (ROT_EARLY && wave == 0 && fi < M && n0 + fg * 4 < N && fg * 4 < th) {
         const int n = n0 + fg * 4;
         const int head = n / ex.hd, d = n - head * ex.hd;
         rot_pos = ex.tok_pos[fi];
@@ -514,7 +517,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         if (MODE == 4) {
             // columns n0 + 4 fg .. +3 of token m: two rotary pairs of one head
             const int n = n0 + fg * 4;
-            if (n >= N) continue;
+            if (n >= N || fg * 4 >= th) continue;        // th is a multiple of 4 here
             const int hd = ex.hd, head = n / hd, d = n - head * hd;
             const int pos = ROT_EARLY ? rot_pos : ex.tok_pos[m];
             float v[4] = {acc[0][ct][0], acc[0][ct][1], acc[0][ct][2], acc[0][ct][3]};
@@ -573,7 +576,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + fg * 4 + j;
-                if (n < N) skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
+                if (n < N && fg * 4 + j < th)
+                    skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
             }
         }
     }
@@ -584,13 +588,57 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     }
 }
 
+// Compute units of the current device (asked once).
+static int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        hipGetDevice(&dev);
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        cus = n > 0 ? n : 1;
+    }
+    return cus;
+}
+
+// Rows of W per workgroup (8..16, in steps of `step`) for a product with N output columns:
+// the height at which the compute unit with the most tiles streams the fewest rows - with
+// 16 rows, 6144 columns are 384 tiles on 256 compute units, half of which stream twice as
+// much as the others; with 12 rows they are 512, two each.  The taller tile on a tie.
+static int pick_tile_rows(int N, int step) {
+    const int cus = compute_units();
+    const long tiles16 = (N + 15) / 16;
+    const long cost16 = ((tiles16 + cus - 1) / cus) * 16;
+    int best = 16;
+    long best_cost = cost16;
+    for (int th = 16 - step; th >= 8; th -= step) {
+        const long tiles = (N + th - 1) / th;
+        const long cost = ((tiles + cus - 1) / cus) * th;
+        if (cost < best_cost) {
+            best = th;
+            best_cost = cost;
+        }
+    }
+    // a lower tile costs a little by itself (more workgroups, shorter runs of rows per load):
+    // it has to save a twentieth of the rows the busiest compute unit streams
+    return best_cost * 20 <= cost16 * 19 ? best : 16;
+}
+
+// Tile height the launcher below uses for this mode and width (the two-kernel norm's
+// shares are one record per tile, so its callers size their buffers by it).
+extern "C" int gfa_skinny_tile_rows(int mode, int N) {
+    return pick_tile_rows(N, (mode == 2 || mode == 4) ? 4 : 1);
+}
+
 template <int MODE>
 static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
                               int ldo, int gate_rows, const SkinnyExtra& ex, hipStream_t stream) {
     constexpr int RT = (MODE == 3) ? 2 : 1;
-    const int tiles = (N + 15) / 16;
-    const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
     const int ct = (M + 15) / 16;
+    // the epilogues that add into the residual stream or rotate pairs work on groups of
+    // four columns: their tiles are 8, 12 or 16 rows high
+    const int th = ct == 1 ? gfa_skinny_tile_rows(MODE, N) : 16;
+    const int tiles = (N + th - 1) / th;
+    const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
     int nw = 1;                                          // waves per tile: aim at >= 2048 waves,
     const int nw_max = (MODE == 3) ? 4 : 8;
     // at least four waves per tile where K allows: one wave walking sixteen rows alone
@@ -618,7 +666,7 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, XPV, XFV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, exl); \
+        skinny_mfma_kernel<CTV, MODE, XPV, XFV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, th, exl); \
     } while (0)
     switch (ct) {
         case 1:                                          // columns of the x operand that stand
@@ -687,9 +735,9 @@ extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t
 }
 
 // residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
-// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [(N + 15) / 16, share_rows] = the
-// workgroups' shares of the rows' sums of squares; share_rows = gfa_share_rows(M).  N a
-// multiple of 4.
+// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [tiles, share_rows] = the
+// workgroups' shares of the rows' sums of squares, tiles = N / gfa_skinny_tile_rows(2, N)
+// rounded up; share_rows = gfa_share_rows(M).  N a multiple of 4.
 extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* residual, int M,
                                           int N, int K, const float* next_g, void* xg_out,
                                           float* ssq_out, hipStream_t stream) {

@@ -88,7 +88,7 @@ def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
                       next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
     ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, R]: per
-    workgroup (16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
+    workgroup (a tile of 8 to 16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
     record (the least that holds M).  Up to 16 rows."""
     _check_operands(x, w, "skinny_into_chain")
     M, K = x.shape
@@ -101,7 +101,8 @@ def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
     if not can_chain_norm(M, N, K):
         raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
     xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    ssq = torch.empty(((N + 15) // 16, share_rows(M)), dtype=torch.float32, device=x.device)
+    th = library("gemm_bf16").gfa_skinny_tile_rows(_i(2), _i(N))     # one record per tile of columns
+    ssq = torch.empty(((N + th - 1) // th, share_rows(M)), dtype=torch.float32, device=x.device)
     check(library("gemm_bf16").gfa_skinny_into_chain_bf16(
         ptr(x), ptr(w), ptr(residual), _i(M), _i(N), _i(K), ptr(next_g), ptr(xg), ptr(ssq),
         stream_handle()), "skinny_into_chain")

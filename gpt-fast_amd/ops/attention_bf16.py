@@ -80,3 +80,4 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
         _i(hd), _f(scale), _i(window), _i(rt), _i(nw), _i(tiles), _i(splits), stream_handle()),
         "attention_bf16")
     return out
+

@@ -21,10 +21,33 @@ from .library import KernelError
 # matrix-core tile of x); beyond that x no longer fits a wave's registers and the vendor
 # library's tiled kernels are faster (measured at 32 and 64 rows)
 SKINNY_MAX_ROWS = 16
-# rows up to which the 17..64-row kernel with the gate in its epilogue beats the vendor
-# library's product followed by the gate kernel (measured: 49 against 54 us at 32 rows of the
-# 8B shape, 56 against 54 at 64)
-WIDE_GATED_MAX_ROWS = 32
+
+
+_units = {}
+
+
+def _compute_units(device) -> int:
+    n = _units.get(device)
+    if n is None:
+        n = _units[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    return n
+
+
+def _own_gate_is_faster(M: int, inner: int, K_: int, device) -> bool:
+    """17..64 rows through the gate: the hand-written kernel (the gate in its epilogue) against
+    the vendor library's product followed by the gate kernel.  A workgroup of the own kernel
+    takes 64 gate columns, so what decides is how the ``inner / 64`` workgroups fill the chip
+    (measured at 17..64 rows): with fewer than four fifths of the compute units (inner 11008:
+    172 on 256) the library wins by 1-8 us at every row count; from there on the own kernel
+    wins by 5-7 us up to 48 rows (inner 14336: 46-52 us against 52-59), and at more rows only
+    where every compute unit has a workgroup and a half or more (inner 28672: 173 against 192
+    us at 64 rows, while inner 14336 loses 55 to 51)."""
+    if K_ % 8 or not 16 < M <= _wide().MAX_ROWS:
+        return False
+    wgs, cus = (inner + 63) // 64, _compute_units(device)
+    if wgs * 5 < cus * 4:
+        return False
+    return M <= 48 or wgs * 2 >= cus * 3
 
 
 def _fast():
@@ -125,7 +148,7 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
         return K.silu_mul(K.gemm_f32(x, w13))
     if x.shape[0] <= SKINNY_MAX_ROWS:
         return _fast().skinny_gated(x, w13)
-    if x.shape[0] <= WIDE_GATED_MAX_ROWS and x.shape[1] % 8 == 0 and w13.shape[0] % 2 == 0:
+    if w13.shape[0] % 2 == 0 and _own_gate_is_faster(x.shape[0], w13.shape[0] // 2, x.shape[1], x.device):
         return _wide().product_gated(x, w13)
     return K.silu_mul(torch.matmul(x, w13.t()))
 

@@ -11,7 +11,8 @@ generate.py:222).  ``--prompt`` is text, or an integer N for a synthetic prompt 
 random token ids below min(1024, vocabulary) as in generate.py:325-327.  Flags of the
 reference that have no meaning here (--compile, --compile_prefill: the kernels are
 compiled ahead of time) are accepted and ignored; those of features outside this
-library (--interactive, --speculate_k, --draft_checkpoint_path) are refused.
+library (--speculate_k, --draft_checkpoint_path) are refused.  ``--interactive`` asks for
+every sample's prompt and writes its text as it is drawn (generate.py:356-377).
 """
 import argparse
 import json
@@ -30,6 +31,10 @@ from .step import Engine
 from .tokenizer import encode_tokens, get_tokenizer
 
 
+B_INST, E_INST = "[INST]", "[/INST]"          # generate.py:270
+INTERACTIVE_POSITIONS = 350                   # generate.py:161
+
+
 def _int_or_str(x):
     try:
         return int(x)
@@ -44,7 +49,7 @@ def build_parser() -> argparse.ArgumentParser:
                    help="Input prompt. If it's an integer, will instead generate a synthetic prompt.")
     p.add_argument("--prompt_ids", type=str, default=None,
                    help="Comma-separated token ids to use as the prompt instead of --prompt.")
-    p.add_argument("--interactive", action="store_true", help="(not available)")
+    p.add_argument("--interactive", action="store_true", help="Whether to launch in interactive mode")
     p.add_argument("--num_samples", type=int, default=5, help="Number of samples.")
     p.add_argument("--max_new_tokens", type=int, default=200, help="Maximum number of new tokens.")
     p.add_argument("--batch_size", type=int, default=1, help="Batch size to benchmark with")
@@ -77,9 +82,16 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
          temperature: float = 0.8, checkpoint_path: Optional[Path] = None,
          random: Optional[str] = None, seed: int = 1234, dtype: str = "bfloat16",
          max_seq_length: Optional[int] = None, profile: Optional[Path] = None,
-         device: str = "cuda", architecture_name: Optional[str] = None, out=print) -> dict:
+         device: str = "cuda", architecture_name: Optional[str] = None, out=print,
+         interactive: bool = False, input_fn=input, stream=None) -> dict:
     """Generates samples and reports throughput the way the reference's ``main`` does
-    (generate.py:272-437).  Returns the aggregate numbers it printed."""
+    (generate.py:272-437).  Returns the aggregate numbers it printed.
+
+    ``interactive``: every sample asks for its prompt (``input_fn``) and its text is written
+    to ``stream`` as it is drawn, four tokens at a time (generate.py:356-377); a folder whose
+    path contains "chat" gets the prompt wrapped in [INST] .. [/INST] (generate.py:298, 359);
+    prompt and new tokens share ``max_seq_length`` positions, 350 unless given
+    (generate.py:160-161)."""
     if (checkpoint_path is None) == (random is None):
         raise SystemExit("give either --checkpoint_path MODEL_FOLDER or --random PRESET")
     device = "cuda:0" if device == "cuda" else device
@@ -114,8 +126,17 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
     prompt_length = prompt if encoded is None else len(encoded)
     if prompt_length < 1:
         raise SystemExit("the prompt needs at least one token")
+    is_chat = checkpoint_path is not None and "chat" in str(checkpoint_path)
+    if interactive:
+        if tokenizer is None:
+            raise SystemExit("--interactive needs a text prompt and a model folder with a tokenizer")
+        if stream is None:
+            stream = sys.stdout
+        max_seq_length = max_seq_length or INTERACTIVE_POSITIONS
     per_seq = max_seq_length or (prompt_length + max_new_tokens)
     per_seq = (per_seq + 63) // 64 * 64
+    if interactive:
+        max_new_tokens = max(1, min(max_new_tokens, per_seq - prompt_length))
     if prompt_length + max_new_tokens > per_seq:
         raise SystemExit(f"prompt ({prompt_length}) + max_new_tokens ({max_new_tokens}) exceed "
                          f"--max_seq_length {per_seq}")
@@ -145,11 +166,27 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
         if profile is not None and i == num_samples - 1:
             prof = torch.profiler.profile()
             prof.__enter__()
+        new_tokens = max_new_tokens
+        callback = None
+        if interactive and i >= 0:
+            text = input_fn("What is your prompt? ")
+            if is_chat:
+                text = f"{B_INST} {text.strip()} {E_INST}"
+            encoded = encode_tokens(tokenizer, text, bos=True)
+            if len(encoded) >= per_seq:
+                out(f"The prompt has {len(encoded)} tokens; {per_seq} positions are there for "
+                    f"prompt and answer (--max_seq_length)")
+                continue
+            new_tokens = min(max_new_tokens, per_seq - len(encoded))
+            callback = _streamer(tokenizer, stream)
         t0 = time.perf_counter()
-        result = generate(engine, [encoded] * batch_size, max_new_tokens,
-                          temperature=temperature, top_k=top_k, seed=seed + max(i, 0))
+        result = generate(engine, [encoded] * batch_size, new_tokens,
+                          temperature=temperature, top_k=top_k, seed=seed + max(i, 0),
+                          callback=callback)
         torch.cuda.synchronize()
         t = time.perf_counter() - t0
+        if callback is not None:
+            callback.flush()
         if prof is not None:
             prof.__exit__(None, None, None)
             prof.export_chrome_trace(f"{profile}.json")
@@ -159,7 +196,10 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
         if batch_size > 1:
             out("Only displaying the first generation of the batch")
         seq = encoded + result.tokens[0]
-        out(tokenizer.decode(seq) if tokenizer is not None else " ".join(map(str, seq)))
+        if interactive:
+            out("")                                       # the text has been streamed, generate.py:404-407
+        else:
+            out(tokenizer.decode(seq) if tokenizer is not None else " ".join(map(str, seq)))
         generated = len(result.tokens[0])
         tps = generated / t
         tokens_per_sec.append(tps)
@@ -183,10 +223,39 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
     return {"tokens_per_sec": mean, "result": result}
 
 
+class _streamer:
+    """Writes a request's text as its tokens are drawn, four at a time (generate.py:362-377).
+    A token is decoded behind a token of known text and that text is cut off again, so that
+    a tokenizer that drops the space in front of a first word keeps it here (the reference
+    does this with the id of '.')."""
+
+    def __init__(self, tokenizer, stream, every: int = 4):
+        self.tokenizer, self.stream, self.every = tokenizer, stream, every
+        lead = tokenizer.encode(".")
+        self.lead = lead[:1]
+        self.cut = len(tokenizer.decode(self.lead)) if self.lead else 0
+        self.buffer: List[str] = []
+        self.done = False
+
+    def __call__(self, rows, tokens) -> None:
+        if self.done or 0 not in rows:
+            return
+        token = tokens[rows.index(0)]
+        self.buffer.append(self.tokenizer.decode(self.lead + [token])[self.cut:])
+        if token == self.tokenizer.eos_id():
+            self.done = True
+        if len(self.buffer) == self.every or self.done:
+            self.flush()
+
+    def flush(self) -> None:
+        if self.buffer:
+            self.stream.write("".join(self.buffer))
+            self.stream.flush()
+            self.buffer.clear()
+
+
 def cli(argv=None) -> int:
     args = build_parser().parse_args(argv)
-    if args.interactive:
-        raise SystemExit("--interactive is not part of this library")
     if args.speculate_k is not None or args.draft_checkpoint_path is not None:
         raise SystemExit("speculative decoding is not part of this library")
     prompt = args.prompt
@@ -194,5 +263,6 @@ def cli(argv=None) -> int:
         prompt = [int(t) for t in args.prompt_ids.split(",")]
     main(prompt, args.num_samples, args.max_new_tokens, args.batch_size, args.top_k,
          args.temperature, args.checkpoint_path, args.random, args.seed, args.dtype,
-         args.max_seq_length, args.profile, args.device, args.architecture)
+         args.max_seq_length, args.profile, args.device, args.architecture,
+         interactive=args.interactive)
     return 0

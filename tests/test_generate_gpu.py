@@ -580,7 +580,7 @@ def test_command_line_random_weights_and_a_batch(tmp_path):
 def test_command_line_refusals(tmp_path_factory):
     folder = util.make_folder(tmp_path_factory.getbasetemp(), "A")
     for args, needle in (
-            (["--checkpoint_path", folder, "--interactive"], "interactive"),
+            (["--checkpoint_path", folder, "--interactive", "--prompt", 5], "interactive"),
             (["--checkpoint_path", folder, "--speculate_k", 4], "speculative"),
             (["--prompt", 4], "either --checkpoint_path"),
             (["--checkpoint_path", folder, "--random", "7B"], "either --checkpoint_path"),
@@ -618,3 +618,39 @@ def test_command_line_text_prompt_starts_with_bos(tmp_path_factory, tmp_path):
     assert "Prompt Length: 4" in proc.stdout
     text = " ".join(f"w{t}" for t in [7, 21, 5, 300] + want)
     assert text in proc.stdout
+
+
+def test_command_line_interactive_streams_the_answer(tmp_path_factory, tmp_path):
+    """--interactive (generate.py:356-377, 404-407): the prompt is asked for, a folder with
+    "chat" in its path wraps it in [INST] .. [/INST] (generate.py:298, 359), and the drawn
+    tokens' text is written as it comes, each word with the space in front of it."""
+    import json as _json
+    import shutil
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    src = util.make_folder(tmp_path_factory.getbasetemp(), "B")
+    for name, wrap in (("plain_folder", False), ("tiny-chat-folder", True)):
+        folder = str(tmp_path / name)
+        shutil.copytree(src, folder)
+        cfg_path = os.path.join(folder, "config.json")
+        c = _json.load(open(cfg_path))
+        c["bos_token_id"] = 7
+        _json.dump(c, open(cfg_path, "w"))
+        vocab = {f"w{i}": i for i in range(c["vocab_size"] - 3)}
+        vocab.update({"[INST]": c["vocab_size"] - 3, "[/INST]": c["vocab_size"] - 2, ".": c["vocab_size"] - 1})
+        tk = Tokenizer(models.WordLevel(vocab, unk_token="w0"))
+        tk.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+        tk.save(os.path.join(folder, "tokenizer.json"))
+        pcfg, w = plain.load_folder(folder)
+        ids = [21, 5, 300]
+        if wrap:
+            ids = [vocab["[INST]"]] + ids + [vocab["[/INST]"]]
+        want = plain.greedy_generate(w, pcfg, [7] + ids, 6)
+        proc = subprocess.run([sys.executable, "-m", "gpt_fast_amd", "--checkpoint_path", folder,
+                               "--interactive", "--temperature", "0", "--num_samples", "1",
+                               "--max_new_tokens", "6", "--dtype", "float32", "--prompt", "w1 w2"],
+                              cwd=ROOT, input="w21 w5 w300\n", capture_output=True, text=True, timeout=110)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert "What is your prompt? " in proc.stdout
+        inv = {i: t for t, i in vocab.items()}
+        assert "".join(" " + inv[t] for t in want) in proc.stdout, proc.stdout[-800:]
+        assert f"Prompt Length: 3" in proc.stdout          # of the warm-up prompt, BOS included

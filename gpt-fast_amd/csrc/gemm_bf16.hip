@@ -263,7 +263,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     constexpr int RT = (MODE == 3) ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
-    // th (8..16) rows of W per workgroup: the host picks it so that the tiles divide evenly
+    // th (12..16) rows of W per workgroup: the host picks it so that the tiles divide evenly
     // over the compute units; operand rows th..15 repeat row th - 1 and are never stored
     const int n0 = blockIdx.x * th;
     char* stage = smem + (size_t)wave * (RT * SM_TILE);
@@ -600,17 +600,19 @@ static int compute_units() {
     return cus;
 }
 
-// Rows of W per workgroup (8..16, in steps of `step`) for a product with N output columns:
+// Rows of W per workgroup (12..16, in steps of `step`) for a product with N output columns:
 // the height at which the compute unit with the most tiles streams the fewest rows - with
 // 16 rows, 6144 columns are 384 tiles on 256 compute units, half of which stream twice as
-// much as the others; with 12 rows they are 512, two each.  The taller tile on a tie.
+// much as the others; with 12 rows they are 512, two each.  The taller tile on a tie.  Not
+// below 12: every tile reads all of x, so lower tiles cost in x what they save in W (10240
+// columns at 8 rows, 1280 tiles for 640, measured 54 against 41 us at 16 rows of x).
 static int pick_tile_rows(int N, int step) {
     const int cus = compute_units();
     const long tiles16 = (N + 15) / 16;
     const long cost16 = ((tiles16 + cus - 1) / cus) * 16;
     int best = 16;
     long best_cost = cost16;
-    for (int th = 16 - step; th >= 8; th -= step) {
+    for (int th = 16 - step; th >= 12; th -= step) {
         const long tiles = (N + th - 1) / th;
         const long cost = ((tiles + cus - 1) / cus) * th;
         if (cost < best_cost) {
@@ -635,7 +637,7 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     constexpr int RT = (MODE == 3) ? 2 : 1;
     const int ct = (M + 15) / 16;
     // the epilogues that add into the residual stream or rotate pairs work on groups of
-    // four columns: their tiles are 8, 12 or 16 rows high
+    // four columns: their tiles are 12 or 16 rows high
     const int th = ct == 1 ? gfa_skinny_tile_rows(MODE, N) : 16;
     const int tiles = (N + th - 1) / th;
     const int pieces = (K + SM_SUBK - 1) / SM_SUBK;

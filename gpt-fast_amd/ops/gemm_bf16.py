@@ -88,7 +88,7 @@ def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
                       next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
     ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, R]: per
-    workgroup (a tile of 8 to 16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
+    workgroup (a tile of 12 to 16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
     record (the least that holds M).  Up to 16 rows."""
     _check_operands(x, w, "skinny_into_chain")
     M, K = x.shape

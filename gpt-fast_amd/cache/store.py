@@ -55,8 +55,10 @@ class KVGroup:
         self.need = need
         self.entries = entries
         self.n_pages = n_pages
-        # keys as rows [PAGE, head_dim]; values transposed [head_dim, PAGE]: the operand
-        # layouts of the matrix-core attention kernel
+        # Every (page, kv head) owns PAGE * head_dim elements of keys and as many of values.
+        # The last two dimensions only give that size: inside, the kernels keep the elements
+        # in the order in which the matrix-core attention reads its operands (csrc/common.h:
+        # key_offset, value_offset), and nothing in Python looks inside.
         # one page beyond the pool (index n_pages) belongs to no sequence: rows of a batch
         # that only fill a fixed shape are pointed at it
         self.k = torch.empty((entries, n_pages + 1, need.n_kv_heads, PAGE, need.head_dim),

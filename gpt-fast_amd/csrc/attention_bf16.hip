@@ -35,7 +35,13 @@ union Frag {
 
 #define LOG2E 1.4426950408889634f
 
-template <int DS, int RT, bool PREFETCH>
+// SINGLE: every sequence brings exactly one token and a kv head's group fits one 16-row tile.
+// The grid is then (splits, kv heads, sequences) and nothing in the kernel's first round of
+// loads depends on another load: the query rows (row of sequence s = s), the sequence's
+// position and the first 63 entries of its page row - one per lane, handed out by readlane
+// as the blocks come - are requested together, and the keys and values follow in the second
+// round.  Otherwise q_start -> position -> page number -> keys is a chain of four.
+template <int DS, int RT, bool PREFETCH, bool SINGLE = false>
 __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
@@ -44,17 +50,39 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows) {
     constexpr int DT = DS * 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    static_assert(!SINGLE || RT == 1, "one token per sequence is one tile of rows");
+    const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    // SINGLE: lane i < 63 holds entry i of the page row and lane 63 the sequence's position,
+    // from one load instruction that needs only arguments which arrive in registers; it is
+    // issued before anything waits for the arguments that are loaded
+    int first_pages = 0;
+    if (SINGLE) {
+        const int* row = table + (size_t)blockIdx.z * table_stride;
+        const int* src = lane == 63 ? start_pos + blockIdx.z : row + (lane < table_stride ? lane : table_stride - 1);
+        first_pages = *src;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int g = blockIdx.y;
-    const int seq = blockIdx.z / n_splits, split = blockIdx.z - seq * n_splits;
     const int R = H / Hkv;
-    const int q0 = q_start[seq];
-    const int rows_total = (q_start[seq + 1] - q0) * R;
-    const int row0 = blockIdx.x * 16 * RT;
-    if (row0 >= rows_total) return;                      // the whole workgroup leaves
-    const int spos = start_pos[seq];
+    int seq, split, q0, rows_total, row0;
+    if (SINGLE) {
+        seq = blockIdx.z;
+        split = blockIdx.x;
+        q0 = seq;
+        rows_total = R;
+        row0 = 0;
+    } else {
+        seq = blockIdx.z / n_splits;
+        split = blockIdx.z - seq * n_splits;
+        q0 = q_start[seq];
+        rows_total = (q_start[seq + 1] - q0) * R;
+        row0 = blockIdx.x * 16 * RT;
+        if (row0 >= rows_total) return;                  // the whole workgroup leaves
+    }
     const int* pages = table + (size_t)seq * table_stride;
+    const int spos = SINGLE ? __builtin_amdgcn_readlane(first_pages, 63) : start_pos[seq];
 
     Frag qf[RT][DS];
     int rpos[RT];             // position of this lane's row in tile rt, -1 if there is none
@@ -63,7 +91,7 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
     for (int rt = 0; rt < RT; ++rt) {
         const int r = row0 + rt * 16 + li;
         const bool valid = r < rows_total;
-        const int t = valid ? r / R : 0, hh = valid ? r - (r / R) * R : 0;
+        const int t = (valid && !SINGLE) ? r / R : 0, hh = valid ? r - t * R : 0;
         rpos[rt] = valid ? spos + t : -1;
         orow[rt] = (size_t)(q0 + t) * H + g * R + hh;
         const bf16_t* qrow = q + orow[rt] * hd;
@@ -74,11 +102,12 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         }
     }
     const int last_row = (row0 + 16 * RT - 1 < rows_total - 1) ? row0 + 16 * RT - 1 : rows_total - 1;
-    const int pmin = spos + row0 / R, pmax = spos + last_row / R;
+    const int pmin = SINGLE ? spos : spos + row0 / R, pmax = SINGLE ? spos : spos + last_row / R;
     const int lo = (window > 0 && pmin - window + 1 > 0) ? pmin - window + 1 : 0;
     const int kb_lo = lo >> 5, nkb = (pmax >> 5) - kb_lo + 1;
-    const int kb_begin = kb_lo + (int)((long)split * nkb / n_splits);
-    const int kb_end = kb_lo + (int)((long)(split + 1) * nkb / n_splits);
+    // 32-bit: a sequence has at most table_stride * 2 blocks, the host checks that times splits
+    const int kb_begin = kb_lo + (int)((unsigned)(split * nkb) / (unsigned)n_splits);
+    const int kb_end = kb_lo + (int)((unsigned)((split + 1) * nkb) / (unsigned)n_splits);
 
     float m[RT], l[RT];
     floatx4_t o[RT][DT];
@@ -92,32 +121,32 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 
     // Row r of key tile kt stands for key 8 (r / 4) + 4 kt + r % 4 of the block, so that the
     // eight scores a lane holds (rows 4 lg .. +3 of both tiles) belong to the eight
-    // consecutive keys 8 lg .. +7 and its value operand is one 16-byte load.
-    // keys: tile kt, row li -> that key, dims ds * 32 + lg * 8 .. +7
+    // consecutive keys 8 lg .. +7 and its value operand is one 16-byte load.  The cache keeps
+    // keys and values in this order (common.h):
+    // keys: tile kt, row li -> slot 16 kt + li of the block, dims ds * 32 + lg * 8 .. +7
     // values: dims dt * 16 + li, keys 8 lg .. +7 of the block
     auto load_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
-        const int page = pages[kb >> 1];
-        const int in_page = (kb & 1) * 32;
-        const bf16_t* kbase = k_pages + page_row(page, g, in_page, Hkv, hd);
+        int page;
+        if (SINGLE && (kb >> 1) < 63) page = __builtin_amdgcn_readlane(first_pages, kb >> 1);
+        else page = pages[kb >> 1];
+        // Every lane loads; for dims beyond the head it is chunk 0 or tile 0, which meets zeros
+        // in the query's operand or goes into accumulators that are never stored.  No load
+        // runs under a branch or a partial execution mask (a choice between the loaded value
+        // and zero would be turned into one), so the waits can count requests.  In the
+        // cache's layout a load instruction reads consecutive lines: 4 x 256 bytes of keys
+        // (16 slots of a chunk each), 1 KB of values.
+        const bf16_t* kbase = k_pages + cache_region(page, g, Hkv, hd) + (size_t)(kb & 1) * 32 * hd;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) {
-                // every lane loads (dims beyond the head: the row's first chunk), then those
-                // lanes are cleared: no load runs under a partial execution mask
                 const int d = ds * 32 + lg * 8;
-                const uint4 got = *(const uint4*)(kbase + (size_t)(8 * (li >> 2) + 4 * kt + (li & 3)) * hd + (d < hd ? d : 0));
-                kf[kt][ds].u = (d < hd) ? got : make_uint4(0, 0, 0, 0);
+                kf[kt][ds].u = *(const uint4*)(kbase + (d < hd ? d >> 3 : 0) * 256 + (kt * 16 + li) * 8);
             }
+        const bf16_t* vbase = v_pages + cache_region(page, g, Hkv, hd) + (kb & 1) * 512 + lane * 8;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const int d = dt * 16 + li;
-            if (d < hd) {
-                vf[dt].u = *(const uint4*)(v_pages + value_elem(page, g, d, in_page + lg * 8, Hkv, hd));
-            } else {
-                vf[dt].u = make_uint4(0, 0, 0, 0);
-            }
-        }
+        for (int dt = 0; dt < DT; ++dt)
+            vf[dt].u = *(const uint4*)(vbase + (dt * 16 < hd ? dt : 0) * 1024);
     };
     auto compute_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
         const int key0 = kb * 32 + lg * 8;                 // this lane's keys: key0 .. key0 + 7
@@ -179,8 +208,8 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
             // the running maximum rarely moves after the first blocks: skip the rescale then
             const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
 #pragma unroll
-            // every tile of dims is multiplied, also those beyond the head (their values are
-            // zero and never stored): with a branch on the head size between the matrix
+            // every tile of dims is multiplied, also those beyond the head (their results are
+            // never stored): with a branch on the head size between the matrix
             // instructions, the two-tile kernel with prefetch gave wrong sums for its first
             // tile at head size 16 once a second block of keys was read
             for (int dt = 0; dt < DT; ++dt) {
@@ -203,6 +232,20 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
                 if (kb + 2 * nw < kb_end) load_block(kb + 2 * nw, kfa, vfa);
                 compute_block(kb + nw, kfb, vfb);
             }
+        }
+    } else if (SINGLE) {
+        // Two blocks in flight: a block's keys and values are requested before the block
+        // ahead of it is multiplied.  Every load is issued unconditionally - a block beyond
+        // the wave's share stands for the share's last one (or the context's first) and is
+        // not multiplied - so that the waits count requests instead of draining them all.
+        Frag kfa[2][DS], vfa[DT], kfb[2][DS], vfb[DT];
+        const int kb_safe = kb_end > kb_lo ? kb_end - 1 : kb_lo;
+        load_block(kb < kb_end ? kb : kb_safe, kfa, vfa);
+        for (; kb < kb_end; kb += 2 * nw) {
+            load_block(kb + nw < kb_end ? kb + nw : kb_safe, kfb, vfb);
+            compute_block(kb, kfa, vfa);
+            load_block(kb + 2 * nw < kb_end ? kb + 2 * nw : kb_safe, kfa, vfa);
+            if (kb + nw < kb_end) compute_block(kb + nw, kfb, vfb);
         }
     } else {
         Frag kfa[2][DS], vfa[DT];
@@ -285,12 +328,10 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 
 // --------------------------------------------------------------------------------------
 // Prompts: a workgroup of four waves owns 128 or 64 query rows (RT tiles of 16 per wave) of
-// one sequence and kv head and walks the keys a page (64 keys) at a time.  A page's keys and values - each
-// one contiguous piece of the cache - are copied by all four waves straight into LDS
-// (global_load_lds, 16 bytes per lane, no registers in between) while earlier pages are
-// multiplied.  An LDS row has no padding; its 16-byte chunks are stored at position
-// (chunk XOR row), chosen on the global side of the copy, so that the operand reads (16
-// rows at a time, the same chunk of each) spread over the banks.
+// one sequence and kv head and walks the keys a page (64 keys) at a time.  A page's keys and
+// values - each one contiguous piece of the cache, already in the operands' order - are
+// copied by all four waves straight into LDS (global_load_lds, 16 bytes per lane, no
+// registers in between) while earlier pages are multiplied.
 //
 // The arithmetic is that of the kernel above, a page (64 keys) at a time.
 // RT row tiles of 16 per wave: 2 (128 rows per workgroup) where the grid exceeds what the chip
@@ -315,10 +356,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     constexpr int DT = DS * 2;
     constexpr int TL_ROWS = TL_WAVES * RT * 16;
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
-    constexpr int KROW = HDM * 2;                         // bytes per key row in LDS
-    constexpr int KCH = HDM / 8;                          // 16-byte chunks per key row
-    constexpr int VROW = 64 * 2;                          // bytes per value row (one dim, 64 keys)
-    constexpr int KBYTES = 64 * KROW, VBYTES = HDM * VROW;
+    constexpr int KBYTES = 64 * HDM * 2, VBYTES = HDM * 64 * 2;   // a page's keys, its values
     constexpr int K_PER = KBYTES / 16 / 256, V_PER = VBYTES / 16 / 256;   // copies per thread
     extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 K tiles, then 2 V tiles
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -385,50 +423,37 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    // Copies.  Thread t fills LDS slots t + 256 i (16 bytes each; a wave's 64 slots are
-    // contiguous, as global_load_lds writes them).  Slot s of a key tile is row s / KCH,
-    // place s % KCH, and holds chunk (place XOR row) of the key that row stands for; keys
-    // are stored in the order the score tiles read them: within a block of 32, key
-    // 8 a + 4 t + b (a < 4, t < 2, b < 4) is row 16 t + 4 a + b, so that the eight scores of
-    // a lane belong to eight consecutive keys (as in the kernel above).  Slot s of a value
-    // tile is dim s / 8, place s % 8, chunk (place XOR dim): keys 8 chunk .. + 7.
-    int k_src[K_PER], v_src[V_PER];                        // byte offsets into the page, -1: nothing
-#pragma unroll
-    for (int i = 0; i < K_PER; ++i) {
-        const int slot = threadIdx.x + i * 256;
-        const int row = slot / KCH, chunk = (slot % KCH) ^ (row & (KCH - 1));
-        const int key = (row & 32) | (((row >> 2) & 3) << 3) | (((row >> 4) & 1) << 2) | (row & 3);
-        k_src[i] = (FULL || chunk * 8 < hd) ? (key * hd + chunk * 8) * 2 : -1;
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER; ++i) {
-        const int slot = threadIdx.x + i * 256;
-        const int dim = slot >> 3, chunk = (slot & 7) ^ (dim & 7);
-        v_src[i] = (FULL || dim < hd) ? dim * VROW + chunk * 16 : -1;
-    }
+    // Copies.  A page's keys and its values lie in the cache in the order in which the operands
+    // are read (common.h), so they are copied as they lie: thread t fills the 16-byte LDS slots
+    // t + 256 i from the same places of the page (a wave's 64 slots are contiguous, as
+    // global_load_lds writes them), and an operand read is 256 consecutive bytes per sixteen
+    // lanes (keys) or 1 KB per wave (values): no two lanes of a pass share a bank.
+    const int hdr = FULL ? HDM : hd;
+    const int page_slots = 8 * hdr;                        // 16-byte slots of keys (of values) per page
     auto copy_keys = [&](int pg) {
-        const char* src = (const char*)(k_pages + page_row(pages[pg], g, 0, Hkv, hd));
+        const char* src = (const char*)(k_pages + cache_region(pages[pg], g, Hkv, hd)) + threadIdx.x * 16;
         char* dst = smem + (pg & 1) * KBYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < K_PER; ++i)
-            if (FULL || k_src[i] >= 0)
+            if (FULL || (int)threadIdx.x + i * 256 < page_slots)
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(src + k_src[i]),
+                    (const __attribute__((address_space(1))) void*)(src + i * 4096),
                     (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
     };
     auto copy_values = [&](int pg) {
-        const char* src = (const char*)(v_pages + value_elem(pages[pg], g, 0, 0, Hkv, hd));
+        const char* src = (const char*)(v_pages + cache_region(pages[pg], g, Hkv, hd)) + threadIdx.x * 16;
         char* dst = smem + 2 * KBYTES + (pg & 1) * VBYTES + wave * 1024;
 #pragma unroll
         for (int i = 0; i < V_PER; ++i)
-            if (FULL || v_src[i] >= 0)
+            if (FULL || (int)threadIdx.x + i * 256 < page_slots)
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(src + v_src[i]),
+                    (const __attribute__((address_space(1))) void*)(src + i * 4096),
                     (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
     };
     // The copies of this thread have arrived.  Slots of the newest page that lie beyond the
     // newest key hold no data yet (whatever the cache held before): their values are set to
-    // zero, by the thread that copied them, so that probability 0 times them is 0.
+    // zero, by the thread that copied them, so that probability 0 times them is 0.  Value slot
+    // s holds keys 32 (s / 64 % 2) + 8 (s / 16 % 4) .. + 7.
     auto copies_landed = [&](int v_pg) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (v_pg > page_hi) return;
@@ -438,24 +463,23 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
             const int slot = threadIdx.x + i * 256;
-            const int chunk = (slot & 7) ^ ((slot >> 3) & 7);
-            if ((FULL || v_src[i] >= 0) && chunk * 8 + 7 > keys_ok) {
+            const int key_first = ((slot >> 6) & 1) * 32 + ((slot >> 4) & 3) * 8;
+            if ((FULL || slot < page_slots) && key_first + 7 > keys_ok) {
                 Frag f;
                 f.u = *(const uint4*)(vt + slot * 16);
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (chunk * 8 + e > keys_ok) f.e[e] = 0;
+                    if (key_first + e > keys_ok) f.e[e] = 0;
                 *(uint4*)(vt + slot * 16) = f.u;
             }
         }
     };
 
-    // operand reads: this lane's row li of a 16-row tile, chunk c at place c XOR row
-    int k_off[DS], v_off[2];
+    // operand reads: keys - chunk ds * 4 + lg of slot 16 t + li of block b, at
+    // b * 64 hd + t * 256 + k_off[ds]; values - tile dt, block hb, at (2 dt + hb) * 1024 + lane * 16
+    int k_off[DS];
 #pragma unroll
-    for (int ds = 0; ds < DS; ++ds) k_off[ds] = li * KROW + (((ds * 4 + lg) ^ (li & (KCH - 1))) << 4);
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) v_off[hb] = li * VROW + (((hb * 4 + lg) ^ (li & 7)) << 4);
+    for (int ds = 0; ds < DS; ++ds) k_off[ds] = (ds * 4 + lg) * 512 + li * 16;
 
     // One page (64 keys) at a time: all scores first, then the softmax of the row tiles, then
     // the second product.  The wave's priority is raised while it issues matrix instructions,
@@ -472,7 +496,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds)
                 kf[ds].u = (FULL || ds * 32 + lg * 8 < hd)
-                               ? *(const uint4*)(kt + kt16 * 16 * KROW + k_off[ds])
+                               ? *(const uint4*)(kt + (kt16 >> 1) * 64 * hdr + (kt16 & 1) * 256 + k_off[ds])
                                : make_uint4(0, 0, 0, 0);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -535,7 +559,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
             for (int hb = 0; hb < 2; ++hb) {
                 Frag vf;
-                vf.u = *(const uint4*)(vt + dt * 16 * VROW + v_off[hb]);
+                vf.u = *(const uint4*)(vt + (dt * 2 + hb) * 1024 + lane * 16);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
                     o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
@@ -701,9 +725,11 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
                              const bf16_t* k, const bf16_t* v, const int* q_start,
                              const int* start_pos, const int* table, int table_stride, bf16_t* out,
                              float* ws_o, float* ws_ml, int H, int Hkv, int hd, float sl2, int window,
-                             int n_splits, int total_rows) {
+                             int n_splits, int total_rows, bool single) {
     const size_t shmem = nw > 1 ? (size_t)(nw - 1) * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
-    if (rt == 1)
+    if (rt == 1 && single)
+        attention_mfma_kernel<DS, 1, false, true><<<dim3(n_splits, grid.y, grid.z / n_splits), 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+    else if (rt == 1)
         attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
     else if (rt == 2)
         attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
@@ -716,13 +742,17 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
 // n_waves (1..4; up to 8 with rt 1) waves per workgroup share the key blocks of their rows;
 // max_tiles = most waves any sequence needs per kv head.  With n_splits > 1, ws_o
 // [n_splits, n_tokens * H, hd] and ws_ml [n_splits, n_tokens * H, 2] hold the partials.
+// one_token_each: the caller vouches that q_start is 0, 1, 2, ... (every sequence one token).
 extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void* v_pages,
                                   const int* q_start, const int* start_pos, const int* table,
                                   int table_stride, void* out, float* ws_o, float* ws_ml,
                                   int n_tokens, int n_seqs, int H, int Hkv, int hd, float scale,
                                   int window, int rt, int n_waves, int max_tiles, int n_splits,
-                                  hipStream_t stream) {
+                                  int one_token_each, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
+    if (one_token_each && n_tokens != n_seqs) return (int)hipErrorInvalidValue;
+    if ((long)table_stride * 2 * (n_splits + 1) >= (1L << 31)) return (int)hipErrorInvalidValue;
+    const bool single = one_token_each && rt == 1 && max_tiles == 1 && H / Hkv <= 16;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || n_splits > 64 || max_tiles < 1 ||
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
         (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > (rt == 1 ? 8 : 4) ||
@@ -735,11 +765,11 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     const bf16_t* kp = (const bf16_t*)k_pages;
     const bf16_t* vp = (const bf16_t*)v_pages;
     if (hd <= 64)
-        launch_attention<2>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<2>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
     else if (hd <= 128)
-        launch_attention<4>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<4>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
     else
-        launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
     if (n_splits > 1)
         attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows);
     return GFA_LAUNCH_RESULT();

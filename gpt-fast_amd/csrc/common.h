@@ -82,19 +82,44 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
-// Address of element (page, kv head, offset in page, 0) of one layer's page pool laid
-// out as [n_pages, n_kv_heads, GFA_PAGE, head_dim].
-__device__ __forceinline__ size_t page_row(int page, int kv_head, int offset, int n_kv_heads,
+// Layout of the cache.  One layer's pool of keys, and its pool of values, gives every
+// (page, kv head) a region of GFA_PAGE * head_dim elements.  Inside a region the elements lie
+// in the order in which the matrix-core attention reads its operands, so that a wave's load
+// instruction covers whole, consecutive cache lines (with keys as rows of head_dim elements,
+// the sixteen rows of an operand tile are sixteen lines, of which a load uses a quarter each:
+// the single-token attention then spends more time on its loads than on anything else).
+//
+// Keys, head sizes that are multiples of 8: [32-key block][chunk of 8 dims][slot][8 dims].
+// The 32 keys of a block fill two 16-row tiles of the score product; key 8 a + 4 t + b
+// (a < 4, t < 2, b < 4) is row 4 a + b of tile t, slot 16 t + 4 a + b: the eight scores a lane
+// receives then belong to eight consecutive keys, which is what the second product wants as
+// its operand.  Other head sizes: rows [key][head_dim].
+__device__ __forceinline__ size_t cache_region(int page, int kv_head, int n_kv_heads, int head_dim) {
+    return ((size_t)page * n_kv_heads + kv_head) * GFA_PAGE * (size_t)head_dim;
+}
+__device__ __forceinline__ int key_slot(int key_in_block) {
+    return ((key_in_block >> 2) & 1) * 16 + (key_in_block >> 3) * 4 + (key_in_block & 3);
+}
+__device__ __forceinline__ int key_offset(int key, int d, int head_dim) {
+    if (head_dim % 8) return key * head_dim + d;
+    return (key >> 5) * 32 * head_dim + (d >> 3) * 256 + key_slot(key & 31) * 8 + (d & 7);
+}
+__device__ __forceinline__ size_t key_elem(int page, int kv_head, int key, int d, int n_kv_heads,
                                            int head_dim) {
-    return (((size_t)page * n_kv_heads + kv_head) * GFA_PAGE + offset) * (size_t)head_dim;
+    return cache_region(page, kv_head, n_kv_heads, head_dim) + key_offset(key, d, head_dim);
 }
 
-// Values are kept transposed: one layer's pool is [n_pages, n_kv_heads, head_dim, GFA_PAGE],
-// so that the keys of a page are contiguous for each element of the head.  The matrix-core
-// attention reads its value operand (8 consecutive keys per lane) straight from this layout.
-__device__ __forceinline__ size_t value_elem(int page, int kv_head, int d, int offset,
-                                             int n_kv_heads, int head_dim) {
-    return (((size_t)page * n_kv_heads + kv_head) * head_dim + d) * GFA_PAGE + offset;
+// Values, head sizes that are multiples of 16: [16-dim tile][32-key block][8-key group][dim][8
+// keys]: the operand of the second product for (tile, block) is 1 KB in lane order (lane
+// 16 g + i: dim i of the tile, keys 8 g .. + 7 of the block).  Other head sizes: transposed
+// rows [dim][GFA_PAGE].
+__device__ __forceinline__ int value_offset(int d, int key, int head_dim) {
+    if (head_dim % 16) return d * GFA_PAGE + key;
+    return (d >> 4) * 1024 + (key >> 5) * 512 + ((key >> 3) & 3) * 128 + (d & 15) * 8 + (key & 7);
+}
+__device__ __forceinline__ size_t value_elem(int page, int kv_head, int d, int key, int n_kv_heads,
+                                             int head_dim) {
+    return cache_region(page, kv_head, n_kv_heads, head_dim) + value_offset(d, key, head_dim);
 }
 
 #define GFA_LAUNCH_RESULT() ((int)hipGetLastError())

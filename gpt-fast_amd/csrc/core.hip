@@ -306,24 +306,22 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
     if (e < qk_slots) {
         const int head = e / half, i = e - head * half;
         const T* src = row + (size_t)head * hd;
-        T* dst;
-        if (head < H) {
-            dst = q_out + ((size_t)n * H + head) * hd;
-        } else {
-            if (!k_pages) return;
-            dst = k_pages + page_row(page, head - H, off, Hkv, hd);
-        }
+        if (head >= H && !k_pages) return;
+        // where element d of this head goes: a row of q_out, or the key's place in its page
+        T* const dst = head < H ? q_out + ((size_t)n * H + head) * hd
+                                : k_pages + cache_region(page, head - H, Hkv, hd);
+        auto place = [&](int d) { return head < H ? d : key_offset(off, d, hd); };
         if (i < rot_pairs) {
             const int ia = layout == 0 ? 2 * i : i;
             const int ib = layout == 0 ? 2 * i + 1 : i + rot_pairs;
             const float a = load_as_float(src + ia), b = load_as_float(src + ib);
             const float c = cs[2 * i], s = cs[2 * i + 1];
-            store_from_float(dst + ia, a * c - b * s);
-            store_from_float(dst + ib, b * c + a * s);
+            store_from_float(dst + place(ia), a * c - b * s);
+            store_from_float(dst + place(ib), b * c + a * s);
         } else {
             const int d0 = rot + 2 * (i - rot_pairs);      // elements rot .. hd-1 are copied
-            dst[d0] = src[d0];
-            dst[d0 + 1] = src[d0 + 1];
+            dst[place(d0)] = src[d0];
+            dst[place(d0 + 1)] = src[d0 + 1];
         }
     } else if (v_pages) {
         const int ev = e - qk_slots;
@@ -374,7 +372,7 @@ __global__ __launch_bounds__(256) void rope_cache_bf16x8_kernel(
         if (head < H) {
             *(uint4*)(q_out + ((size_t)n * H + head) * hd + d0) = out.u;
         } else if (k_pages) {
-            *(uint4*)(k_pages + page_row(page, head - H, off, Hkv, hd) + d0) = out.u;
+            *(uint4*)(k_pages + key_elem(page, head - H, off, d0, Hkv, hd)) = out.u;   // one chunk of 8 dims
         }
     } else if (v_pages) {
         const int g = head - H - Hkv;
@@ -444,9 +442,10 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
         const int j = base + threadIdx.x;
         float s = -INFINITY;
         if (j <= pos) {
-            const T* kr = k_pages + page_row(pages[j / GFA_PAGE], g, j % GFA_PAGE, Hkv, hd);
+            const T* kr = k_pages + cache_region(pages[j / GFA_PAGE], g, Hkv, hd);
             float dot = 0.f;
-            for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], load_as_float(kr + d), dot);
+            for (int d = 0; d < hd; ++d)
+                dot = fmaf(qs[d], load_as_float(kr + key_offset(j % GFA_PAGE, d, hd)), dot);
             s = dot * scale;
         }
         const float m_new = fmaxf(m, block_max(s, scratch));

@@ -545,7 +545,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                     : ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + pos / GFA_PAGE];
                 const int off = pos % GFA_PAGE;
                 if (head < ex.H + ex.Hkv) {
-                    *(uint2*)(ex.k_pages + page_row(page, head - ex.H, off, ex.Hkv, hd) + d) =
+                    *(uint2*)(ex.k_pages + key_elem(page, head - ex.H, off, d, ex.Hkv, hd)) =
                         make_uint2(pk.u.x, pk.u.y);
                 } else {
                     const int g = head - ex.H - ex.Hkv;

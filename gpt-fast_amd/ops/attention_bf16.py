@@ -77,7 +77,8 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
     check(library("attention_bf16").gfa_attention_bf16(
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos), ptr(table),
         _i(table.shape[1]), ptr(out), ptr(ws_o), ptr(ws_ml), _i(n), _i(batch.n_seqs), _i(H), _i(G),
-        _i(hd), _f(scale), _i(window), _i(rt), _i(nw), _i(tiles), _i(splits), stream_handle()),
+        _i(hd), _f(scale), _i(window), _i(rt), _i(nw), _i(tiles), _i(splits),
+        _i(int(batch.max_q_len == 1 and n == batch.n_seqs)), stream_handle()),
         "attention_bf16")
     return out
 

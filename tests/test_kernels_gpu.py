@@ -6,6 +6,8 @@ import math
 import pytest
 import torch
 
+from util import from_cache_order, to_cache_order
+
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
@@ -190,6 +192,7 @@ def _paged(S_list, G, hd, dtype, seed):
             n = min(64, S - 64 * i)
             k_pages[p, :, :n] = k[64 * i:64 * i + n].transpose(0, 1)
             v_pages[p, :, :, :n] = v[64 * i:64 * i + n].permute(1, 2, 0)
+    k_pages, v_pages = to_cache_order(k_pages, v_pages)
     return k_pages.to(DEV), v_pages.to(DEV), table.to(DEV), ks, vs
 
 
@@ -329,6 +332,36 @@ def test_attention_finds_one_far_key():
             close(out[0, h], vs[0][target, h // (H // G)].float(), 2e-2)
 
 
+@pytest.mark.parametrize("H,G,hd,window", [(8, 2, 128, 0), (4, 4, 16, 0), (16, 1, 64, 0), (6, 2, 48, 37),
+                                           (3, 1, 256, 0), (10, 2, 112, 100), (32, 8, 128, 4000)])
+def test_single_token_attention_in_a_batch(H, G, hd, window):
+    """One new token for each sequence of a batch (the step that decoding repeats): lengths
+    from one key to 4,100 in one launch - the last one's page row is longer than the 63
+    entries a wave keeps in registers - on scattered pages with poisoned tails."""
+    from gpt_fast_amd.ops import attention as A
+    lens = [1, 63, 64, 65, 200, 333, 4100, 2]
+    k_pages, v_pages, table, ks, vs = _paged(lens, G, hd, torch.bfloat16, seed=hd + H)
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(len(lens), H, hd, generator=g).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(hd)
+
+    class B:
+        pass
+    batch = B()
+    batch.tok_seq = torch.arange(len(lens), dtype=torch.int32, device=DEV)
+    batch.tok_pos = torch.tensor([S - 1 for S in lens], dtype=torch.int32, device=DEV)
+    batch.n_tokens = batch.n_seqs = len(lens)
+    batch.max_q_len, batch.max_kv_len, batch.is_decode = 1, max(lens), True
+    batch.q_start = torch.arange(len(lens) + 1, dtype=torch.int32, device=DEV)
+    batch.start_pos = batch.tok_pos.clone()
+    batch.host_q_start, batch.host_start_pos = list(range(len(lens) + 1)), [S - 1 for S in lens]
+    out = A.attention(q.to(DEV), k_pages, v_pages, batch, table, scale, window).cpu()
+    assert not torch.isnan(out).any()
+    for b, S in enumerate(lens):
+        ref = _attention_ref(q[b].float(), ks[b].float(), vs[b].float(), S - 1, scale, window)
+        close(out[b], ref, 1.5e-2)
+
+
 @pytest.mark.parametrize("H,G,hd,window", [(8, 2, 128, 0), (4, 4, 64, 0), (6, 2, 96, 0), (8, 2, 128, 1000),
                                            (3, 1, 48, 0)])
 def test_prompt_attention_over_thousands_of_keys(H, G, hd, window, monkeypatch):
@@ -447,7 +480,7 @@ def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):
         ref[:, :H + G, rot // 2:rot] = b * c + a * s
     tol = 2e-4 if dtype == torch.float32 else 1e-2      # float: cos/sin of angles up to 4000
     close(q_out, ref[:, :H], tol)
-    kc, vc = kp.cpu().float(), vp.cpu().float()
+    kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
     for n, p in enumerate(pos):
         page = int(table[0, p // 64])
         close(kc[page, :, p % 64], ref[n, H:H + G], tol)

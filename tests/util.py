@@ -87,3 +87,44 @@ def mixed_step_case(V):
     before = {"d0": 8, "d1": 65, "d2": 129, "c": 70}            # fed by the earlier step
     mixed = {"d0": 1, "d1": 1, "d2": 1, "c": 40, "p": 130}      # fed by the mixed step
     return seqs, before, mixed
+
+
+# The order of a cache page's elements, written down from its description in csrc/common.h
+# (not shared with the kernels: the kernel tests build and read pages through these).
+def key_places(hd):
+    """[64, hd] -> place of element (key, d) inside a (page, kv head) region of keys."""
+    key = torch.arange(64)[:, None].expand(64, hd)
+    d = torch.arange(hd)[None, :].expand(64, hd)
+    if hd % 8:
+        return key * hd + d
+    kk = key % 32                                   # key 8 a + 4 t + b of a block -> slot 16 t + 4 a + b
+    slot = ((kk // 4) % 2) * 16 + (kk // 8) * 4 + kk % 4
+    return (key // 32) * 32 * hd + (d // 8) * 256 + slot * 8 + d % 8
+
+
+def value_places(hd):
+    """[hd, 64] -> place of element (d, key) inside a (page, kv head) region of values."""
+    d = torch.arange(hd)[:, None].expand(hd, 64)
+    key = torch.arange(64)[None, :].expand(hd, 64)
+    if hd % 16:
+        return d * 64 + key
+    return (d // 16) * 1024 + (key // 32) * 512 + ((key // 8) % 4) * 128 + (d % 16) * 8 + key % 8
+
+
+def to_cache_order(k_rows, v_cols):
+    """Pages given as keys [n, G, 64, hd] and values [n, G, hd, 64] -> the same shapes with the
+    elements where the kernels keep them."""
+    n, G, _, hd = k_rows.shape
+    k = torch.empty_like(k_rows).view(n, G, -1)
+    v = torch.empty_like(v_cols).view(n, G, -1)
+    k[..., key_places(hd).reshape(-1)] = k_rows.reshape(n, G, -1)
+    v[..., value_places(hd).reshape(-1)] = v_cols.reshape(n, G, -1)
+    return k.view_as(k_rows), v.view_as(v_cols)
+
+
+def from_cache_order(k_pages, v_pages):
+    """The inverse: what the kernels keep -> keys [n, G, 64, hd], values [n, G, hd, 64]."""
+    n, G, _, hd = k_pages.shape
+    k = k_pages.reshape(n, G, -1)[..., key_places(hd).reshape(-1)].view(n, G, 64, hd)
+    v = v_pages.reshape(n, G, -1)[..., value_places(hd).reshape(-1)].view(n, G, hd, 64)
+    return k, v

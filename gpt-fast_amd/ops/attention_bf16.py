@@ -8,12 +8,18 @@ from .library import KernelError, check, library, ptr, require_contiguous, requi
 _i = ctypes.c_int
 _f = ctypes.c_float
 
-TARGET_WAVES = 2048        # single-token steps split the context until this many waves run
 MAX_SPLITS = 32
-# A wave takes its keys one 32-key block after another, each a round trip to memory; the
-# splits are summed by a second kernel (one wave per row, its loads in flight together), so
-# a wave may be left with as few as 64 keys (measured at contexts of 256 to 16,384 keys).
-KEYS_PER_WAVE = 64
+# Single-token steps.  A wave takes its keys one 32-key block after another (0.6 us each, two
+# in flight); splitting a context over several workgroups shortens that chain but costs a
+# second kernel that sums the splits (3 to 4 us with its boundary).  Measured on contexts of
+# 128 to 16,384 keys and 1 to 64 sequences (8 kv heads, head size 128): no split pays while a
+# wave has at most SPLIT_FROM_BLOCKS blocks; 128 workgroups already stream the cache at the
+# memory's rate, so splits only make up for missing workgroups, never beyond FILL_GROUPS; a
+# split is left with two blocks per wave at least.
+SPLIT_FROM_BLOCKS = 6
+FILL_GROUPS = 256
+STREAMING_GROUPS = 128
+LONG_BLOCKS = 48           # with 128..255 workgroups, two splits from this many blocks per wave on
 
 
 TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
@@ -30,10 +36,15 @@ def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int)
         rt = 1
         nw = 4 if hd <= 128 else 2
         tiles = (R + 15) // 16
-        waves = n_seqs * G * tiles * nw
-        by_keys = table_width * 64 // (KEYS_PER_WAVE * nw)
-        splits = min((TARGET_WAVES + waves - 1) // waves, MAX_SPLITS, by_keys)
-        return rt, nw, tiles, max(splits, 1)
+        groups = n_seqs * G * tiles                      # workgroups without any split
+        blocks = (table_width * 2 + nw - 1) // nw          # key blocks per wave at most
+        if blocks <= SPLIT_FROM_BLOCKS or groups >= FILL_GROUPS:
+            splits = 1
+        elif groups >= STREAMING_GROUPS:
+            splits = 2 if blocks >= LONG_BLOCKS else 1
+        else:
+            splits = min((blocks + 1) // 2, (FILL_GROUPS + groups - 1) // groups, MAX_SPLITS)
+        return rt, nw, tiles, splits
     rt = PREFILL_ROW_TILES if hd <= 128 else min(PREFILL_ROW_TILES, 2)
     rows = max_q_len * R
     if rows <= 16:

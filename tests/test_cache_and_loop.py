@@ -370,20 +370,27 @@ def test_bench_refuses_more_than_one_gpu_in_one_line():
 
 def test_attention_plan_for_single_token_steps():
     """How a single-token step is cut over waves: pure arithmetic, no kernel.  More sequences
-    mean fewer context splits; a split never leaves a wave less than 64 keys of the table's
-    capacity, never exceeds 32, and short contexts are not split at all."""
+    mean fewer context splits; a split leaves a wave two 32-key blocks of the table's capacity
+    at least, there are never more than 32, and short contexts are not split at all."""
     from gpt_fast_amd.ops.attention_bf16 import MAX_SPLITS, plan
     H, G, hd = 32, 8, 128
-    for n_seqs in (1, 3, 8, 64, 300):
-        for width in (1, 4, 17, 65, 257, 2048):
+    for n_seqs in (1, 3, 8, 16, 64, 300):
+        last = MAX_SPLITS
+        for width in (1, 4, 12, 17, 65, 257, 2048):
             rt, nw, tiles, splits = plan(n_seqs, 1, H, G, hd, width)
             assert rt == 1 and tiles == 1 and nw == 4
             assert 1 <= splits <= MAX_SPLITS
-            assert splits == 1 or splits * nw * 64 <= width * 64
-    assert plan(1, 1, H, G, hd, 4)[3] == 1
-    assert plan(1, 1, H, G, hd, 65)[3] == 16 and plan(1, 1, H, G, hd, 257)[3] == 32
-    assert plan(64, 1, H, G, hd, 65)[3] == 1
-    assert plan(8, 1, H, G, hd, 65)[3] == 8
+            assert splits == 1 or splits * nw * 64 <= width * 64 + nw * 64
+        for n_more in (n_seqs, 2 * n_seqs, 5 * n_seqs):
+            now = plan(n_more, 1, H, G, hd, 257)[3]
+            assert now <= last
+            last = now
+    assert plan(1, 1, H, G, hd, 4)[3] == 1 and plan(8, 1, H, G, hd, 12)[3] == 1
+    assert plan(1, 1, H, G, hd, 33)[3] == 9 and plan(1, 1, H, G, hd, 65)[3] == 17
+    assert plan(1, 1, H, G, hd, 257)[3] == 32
+    assert plan(8, 1, H, G, hd, 65)[3] == 4 and plan(4, 1, H, G, hd, 65)[3] == 8
+    assert plan(16, 1, H, G, hd, 65)[3] == 1 and plan(16, 1, H, G, hd, 129)[3] == 2
+    assert plan(64, 1, H, G, hd, 2048)[3] == 1
     # 32 query heads on one kv head: two row tiles per token; wide heads: two waves
     assert plan(2, 1, 32, 1, 64, 8)[2] == 2
     assert plan(2, 1, 4, 2, 256, 8)[1] == 2

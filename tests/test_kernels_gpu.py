@@ -301,7 +301,7 @@ def test_attention_finds_one_far_key():
     """One key among hundreds stands out (its score is scaled up): the output must be
     that key's value, wherever in the cache it lies - first row, a page edge, the last."""
     from gpt_fast_amd.ops import attention as A
-    # 700 keys: two context splits in the single-token kernel; 5000 keys: nineteen, summed by
+    # 700 keys: six blocks per wave, no context split; 5000 keys: twenty splits, summed by
     # the second kernel in batches of eight and a rest; 9000 keys of a small head: thirty-two
     # splits, more than the lanes that hold the head's dims in that kernel; then other head
     # sizes and group sizes (two row tiles per kv head; two waves per workgroup) with splits

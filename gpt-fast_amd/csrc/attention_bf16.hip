@@ -35,6 +35,23 @@ union Frag {
 
 #define LOG2E 1.4426950408889634f
 
+// Maximum (sum) over the four lanes i, i + 16, i + 32, i + 48: the lanes that hold one row's
+// scores.  The swaps exchange rows of sixteen lanes between two registers (odd rows of the
+// first with even rows of the second; the upper half of the first with the lower half of the
+// second), so two copies of a value meet their neighbours without a trip through LDS.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float sum_over_lane_groups(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // SINGLE: every sequence brings exactly one token and a kv head's group fits one 16-row tile.
 // The grid is then (splits, kv heads, sequences) and nothing in the kernel's first round of
 // loads depends on another load: the query rows (row of sequence s = s), the sequence's
@@ -171,6 +188,8 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const bool masked = kb * 32 + 31 > pmin || (window > 0 && kb * 32 < pmax - window + 1);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
+            // raw scores; the scale is positive, so it is applied to the maximum and inside
+            // the exponent's multiply-add instead of to every score
             float sv[8];
             float mx = -INFINITY;
             if (masked) {
@@ -178,19 +197,17 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int key = key0 + e;
-                    const float v = s[rt][e >> 2][e & 3] * scale_log2;
-                    sv[e] = (key <= rpos[rt] && key >= first) ? v : -INFINITY;
+                    sv[e] = (key <= rpos[rt] && key >= first) ? s[rt][e >> 2][e & 3] : -INFINITY;
                     mx = fmaxf(mx, sv[e]);
                 }
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    sv[e] = s[rt][e >> 2][e & 3] * scale_log2;
+                    sv[e] = s[rt][e >> 2][e & 3];
                     mx = fmaxf(mx, sv[e]);
                 }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = max_over_lane_groups(mx) * scale_log2;
             const float m_new = fmaxf(m[rt], mx);
             // a row without any key so far keeps m = -inf: exp2(-inf - -inf) must not be formed
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -199,23 +216,26 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = __builtin_amdgcn_exp2f(sv[e] - m_safe);      // 2^-inf = 0
+                const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], scale_log2, -m_safe));   // 2^-inf = 0
                 sum += p;
                 pf.e[e] = float_to_bf16(p);
             }
             l[rt] = l[rt] * alpha + sum;
             m[rt] = m_new;
             // the running maximum rarely moves after the first blocks: skip the rescale then
-            const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+            // (a real branch: as a choice per element it costs as much as the rescale)
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= alpha;
+            }
 #pragma unroll
             // every tile of dims is multiplied, also those beyond the head (their results are
             // never stored): with a branch on the head size between the matrix
             // instructions, the two-tile kernel with prefetch gave wrong sums for its first
             // tile at head size 16 once a second block of keys was read
-            for (int dt = 0; dt < DT; ++dt) {
-                if (rescale) o[rt][dt] *= alpha;
+            for (int dt = 0; dt < DT; ++dt)
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
-            }
         }
     };
 
@@ -258,8 +278,7 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
     float lt[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        lt[rt] = l[rt] + __shfl_xor(l[rt], 16, 64);
-        lt[rt] += __shfl_xor(lt[rt], 32, 64);
+        lt[rt] = sum_over_lane_groups(l[rt]);
     }
     if (nw > 1) {                 // the waves' partial results meet in LDS, added in wave order
         float* sm_ml = (float*)smem;                                  // [nw - 1][RT][16][2]: waves 1 ..
@@ -653,7 +672,8 @@ extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, cons
                                         int Hkv, int hd, float scale, int window, int max_rows,
                                         int row_tiles, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_rows < 1 || row_tiles < 0 || row_tiles > 2)
+    if (hd % 16 != 0 || hd > 128 || H % Hkv != 0 || max_rows < 1 || row_tiles < 0 || row_tiles > 2 ||
+        !(scale > 0.f))                                   // the kernels take maxima before scaling
         return (int)hipErrorInvalidValue;
     const float sl2 = scale * LOG2E;
     const bf16_t* qp = (const bf16_t*)q;
@@ -754,6 +774,7 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     if ((long)table_stride * 2 * (n_splits + 1) >= (1L << 31)) return (int)hipErrorInvalidValue;
     const bool single = one_token_each && rt == 1 && max_tiles == 1 && H / Hkv <= 16;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || n_splits > 64 || max_tiles < 1 ||
+        !(scale > 0.f) ||                                 // the kernels take maxima before scaling
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
         (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > (rt == 1 ? 8 : 4) ||
         (size_t)(n_waves - 1) * rt * (128 + (hd <= 64 ? 2 : hd <= 128 ? 4 : 8) * 2 * 1024) > 65536)

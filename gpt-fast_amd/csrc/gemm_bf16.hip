@@ -30,9 +30,22 @@ __device__ __forceinline__ float dot8(const Pack8& a, const Pack8& b, float acc)
 
 __device__ __forceinline__ float silu(float a) { return a / (1.f + expf(-a)); }
 
+// Rows kept for a few-row product that reads them next ("chunked", pad = 4, 8 or 16 rows):
+// [columns / 8][pad][8] instead of [rows][columns], so that the sixteen lanes which load one
+// 16-byte chunk each of sixteen different rows read consecutive bytes (whole cache lines)
+// instead of sixteen lines.  Element (m, n) of such rows:
+__device__ __forceinline__ size_t chunked_elem(int m, int n, int pad) {
+    return ((size_t)(n >> 3) * pad + m) * 8 + (n & 7);
+}
+
 template <int MODE>
-__device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, float v, float gate_v) {
+__device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, float v, float gate_v,
+                                             int out_pad = 0) {
     if (MODE == 4) return;                     // the rotary epilogue stores by itself
+    if (MODE == 3 && out_pad) {
+        ((bf16_t*)out)[chunked_elem(m, n, out_pad)] = float_to_bf16(silu(v) * gate_v);
+        return;
+    }
     if (MODE == 0) {
         ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(v);
     } else if (MODE == 1) {
@@ -239,7 +252,7 @@ struct SkinnyExtra {
     const int* table;
     int table_stride, H, Hkv, hd, rot;
     // A norm spread over two kernels (one tile of rows).  The kernel that completes the
-    // residual stream (MODE 2) also writes xg_out [M, N] = bfloat16(new residual * next_g) and
+    // residual stream (MODE 2) also writes xg_out = bfloat16(new residual * next_g) (chunked) and
     // ssq_out [tiles, share_rows] (tiles of gfa_skinny_tile_rows(2, N) columns): each workgroup's share of its rows' sums of squares (float,
     // from the float residual).  The next product takes xg as its x, adds the shares in a fixed
     // order (ssq_in [t_in, share_rows]) and scales its result by rsqrt(sum / K + eps): a factor per row
@@ -251,6 +264,9 @@ struct SkinnyExtra {
     int t_in;
     int share_off;            // byte offset in LDS of the waves' pieces for the shares
     int share_rows;           // rows per share record: 4, 8 or 16 (the least that holds M)
+    // chunked rows (see chunked_elem): x is read so if x_pad > 0; the gate's output (MODE 3)
+    // is written so if out_pad > 0; xg_out always is, with share_rows as its pad
+    int x_pad, out_pad;
 };
 
 // Rows per record of the sums-of-squares shares for M rows of x.
@@ -333,8 +349,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 const int m = XF ? ct * 16 + 8 * (s & 1) + (fi & 7) : ct * 16 + fi % XROWS;
-                xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)(x + (size_t)m * K + kk)
-                                                : make_uint4(0, 0, 0, 0);
+                const bf16_t* src = ex.x_pad ? x + chunked_elem(m, kk, ex.x_pad) : x + (size_t)m * K + kk;
+                xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)src : make_uint4(0, 0, 0, 0);
             }
         }
     };
@@ -569,7 +585,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                 e[1] = float_to_bf16(r.y * g.y);
                 e[2] = float_to_bf16(r.z * g.z);
                 e[3] = float_to_bf16(r.w * g.w);
-                *(uint2*)(ex.xg_out + (size_t)m * ldo + n0 + fg * 4) = make_uint2(pk.u.x, pk.u.y);
+                *(uint2*)(ex.xg_out + chunked_elem(m, n0 + fg * 4, ex.share_rows)) = make_uint2(pk.u.x, pk.u.y);
                 part_ssq = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
             }
         } else {
@@ -577,7 +593,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + fg * 4 + j;
                 if (n < N && fg * 4 + j < th)
-                    skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f);
+                    skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f, ex.out_pad);
             }
         }
     }
@@ -731,42 +747,51 @@ extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t
         ex.t_in = t_in;
         ex.share_rows = gfa_share_rows(M);
         ex.eps = eps;
+        ex.x_pad = ex.share_rows;                         // xg is kept chunked
     }
     const int N = (H + 2 * Hkv) * hd;
     return launch_skinny_mfma<4>((const bf16_t*)x, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
 }
 
 // residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
-// xg_out [M, N] = bfloat16(new residual * next_g), ssq_out [tiles, share_rows] = the
-// workgroups' shares of the rows' sums of squares, tiles = N / gfa_skinny_tile_rows(2, N)
-// rounded up; share_rows = gfa_share_rows(M).  N a multiple of 4.
-extern "C" int gfa_skinny_into_chain_bf16(const void* x, const void* w, float* residual, int M,
-                                          int N, int K, const float* next_g, void* xg_out,
-                                          float* ssq_out, hipStream_t stream) {
+// xg_out = bfloat16(new residual * next_g), kept chunked ([N / 8][share_rows][8], see
+// chunked_elem), ssq_out [tiles, share_rows] = the workgroups' shares of the rows' sums of
+// squares, tiles = N / gfa_skinny_tile_rows(2, N) rounded up; share_rows = gfa_share_rows(M).
+// N a multiple of 8.  x_chunked: x is kept chunked too (pad gfa_share_rows(M)), as the gate
+// of gfa_skinny_after_chain_bf16 leaves its result on request.
+extern "C" int gfa_skinny_into_chain_bf16(const void* x, int x_chunked, const void* w,
+                                          float* residual, int M, int N, int K, const float* next_g,
+                                          void* xg_out, float* ssq_out, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 8 != 0 || N % 4 != 0 || !next_g || !xg_out || !ssq_out)
+    if (M > 16 || K <= 0 || K % 8 != 0 || N % 8 != 0 || !next_g || !xg_out || !ssq_out)
         return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.share_rows = gfa_share_rows(M);
+    ex.x_pad = x_chunked ? ex.share_rows : 0;
     ex.next_g = next_g;
     ex.xg_out = (bf16_t*)xg_out;
     ex.ssq_out = ssq_out;
     return launch_skinny_mfma<2>((const bf16_t*)x, (const bf16_t*)w, residual, M, N, K, N, 0, ex, stream);
 }
 
-// The product that follows: x = xg [M <= 16, K], the result scaled by
-// rsqrt(sum of ssq_in[:, m] / K + eps), ssq_in [t_in, gfa_share_rows(M)].  mode 0 bfloat16
-// out, 1 float out, 3 gate.
+// The product that follows: x = xg (M <= 16 rows of K, chunked as the kernel above leaves
+// them), the result scaled by rsqrt(sum of ssq_in[:, m] / K + eps), ssq_in [t_in,
+// gfa_share_rows(M)].  mode 0 bfloat16 out, 1 float out, 3 gate; out_chunked (gate only, N a
+// multiple of 8): the result is left chunked for the product that reads it next.
 extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, int t_in, float eps,
                                            const void* w, void* out, int M, int N, int K, int ldo,
-                                           int mode, int gate_rows, hipStream_t stream) {
+                                           int mode, int gate_rows, int out_chunked,
+                                           hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K <= 0 || K % 8 != 0 || !ssq_in || t_in <= 0) return (int)hipErrorInvalidValue;
+    if (out_chunked && (mode != 3 || N % 8 != 0)) return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.ssq_in = ssq_in;
     ex.t_in = t_in;
     ex.share_rows = gfa_share_rows(M);
     ex.eps = eps;
+    ex.x_pad = ex.share_rows;
+    ex.out_pad = out_chunked ? ex.share_rows : 0;
     const bf16_t* xp = (const bf16_t*)xg;
     const bf16_t* wp = (const bf16_t*)w;
     switch (mode) {

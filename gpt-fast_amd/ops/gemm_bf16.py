@@ -12,6 +12,43 @@ MAX_ROWS = 64
 DOT_MAX_ROWS = 1
 
 
+class ChunkedRows:
+    """Up to 16 rows of bfloat16 as one few-row product leaves them for the next:
+    ``data`` holds [cols / 8][pad][8] (pad = 4, 8 or 16, the least that holds the rows), so
+    that the lanes which load one 16-byte chunk each of different rows read consecutive
+    bytes.  Only the kernels of this module look inside; :meth:`to_rows` is for tests."""
+
+    __slots__ = ("data", "rows", "cols", "pad")
+
+    def __init__(self, rows: int, cols: int, device):
+        if not 0 < rows <= 16 or cols % 8:
+            raise KernelError(f"chunked rows: {rows} x {cols} (1..16 rows, columns in eights)")
+        self.rows, self.cols, self.pad = rows, cols, share_rows(rows)
+        self.data = torch.empty(cols * self.pad, dtype=torch.bfloat16, device=device)
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def to_rows(self) -> torch.Tensor:
+        t = self.data.view(self.cols // 8, self.pad, 8).permute(1, 0, 2).reshape(self.pad, self.cols)
+        return t[:self.rows].contiguous()
+
+
+def share_rows(n_rows: int) -> int:
+    """Rows per record of the sums-of-squares shares, and per chunk of chunked rows, for this
+    many rows of x."""
+    return 4 if n_rows <= 4 else 8 if n_rows <= 8 else 16
+
+
 def _entry(M: int, K: int):
     lib = library("gemm_bf16")
     if M > DOT_MAX_ROWS and K % 8 == 0:
@@ -79,18 +116,14 @@ def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:
     return 0 < n_rows <= 16 and n_out % 8 == 0 and inner % 8 == 0
 
 
-def share_rows(n_rows: int) -> int:
-    """Rows per record of the sums-of-squares shares for this many rows of x."""
-    return 4 if n_rows <= 4 else 8 if n_rows <= 8 else 16
-
-
-def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
-                      next_g: torch.Tensor):
+def skinny_into_chain(x, w: torch.Tensor, residual: torch.Tensor, next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
-    ``xg`` = bfloat16(new residual * next_g) [M, N] and ``ssq`` float32 [tiles, R]: per
-    workgroup (a tile of 12 to 16 columns) its share of each row's sum of squares, R = 4, 8 or 16 rows per
-    record (the least that holds M).  Up to 16 rows."""
-    _check_operands(x, w, "skinny_into_chain")
+    ``xg`` = bfloat16(new residual * next_g) as :class:`ChunkedRows` and ``ssq`` float32
+    [tiles, R]: per workgroup (a tile of 12 to 16 columns) its share of each row's sum of
+    squares, R = 4, 8 or 16 rows per record (the least that holds M).  Up to 16 rows; x a
+    tensor [M, K] or :class:`ChunkedRows` (the gate's result, left so on request)."""
+    chunked = isinstance(x, ChunkedRows)
+    _check_operands(x.data.view(x.pad, x.cols)[:x.rows] if chunked else x, w, "skinny_into_chain")
     M, K = x.shape
     N = w.shape[0]
     require_device(residual, next_g)
@@ -100,23 +133,25 @@ def skinny_into_chain(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
         raise KernelError("skinny_into_chain: one float32 norm weight per column")
     if not can_chain_norm(M, N, K):
         raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
-    xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    xg = ChunkedRows(M, N, w.device)
     th = library("gemm_bf16").gfa_skinny_tile_rows(_i(2), _i(N))     # one record per tile of columns
-    ssq = torch.empty(((N + th - 1) // th, share_rows(M)), dtype=torch.float32, device=x.device)
+    ssq = torch.empty(((N + th - 1) // th, share_rows(M)), dtype=torch.float32, device=w.device)
     check(library("gemm_bf16").gfa_skinny_into_chain_bf16(
-        ptr(x), ptr(w), ptr(residual), _i(M), _i(N), _i(K), ptr(next_g), ptr(xg), ptr(ssq),
-        stream_handle()), "skinny_into_chain")
+        ptr(x.data if chunked else x), _i(int(chunked)), ptr(w), ptr(residual), _i(M), _i(N), _i(K),
+        ptr(next_g), ptr(xg.data), ptr(ssq), stream_handle()), "skinny_into_chain")
     return xg, ssq
 
 
 def _check_chain(xg, ssq, w, what):
-    _check_operands(xg, w, what)
-    require_device(ssq)
-    if xg.shape[0] > 16 or w.shape[1] % 8:
-        raise KernelError(f"{what}: takes 1..16 rows and an inner size that is a multiple of 8")
-    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[1] != share_rows(xg.shape[0]) \
+    if not isinstance(xg, ChunkedRows):
+        raise KernelError(f"{what}: the first half of the norm comes as ChunkedRows")
+    require_device(xg.data, w, ssq)
+    require_contiguous(w=w)
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != xg.cols or w.shape[1] % 8:
+        raise KernelError(f"{what}: xg {xg.shape} and w {tuple(w.shape)} do not fit")
+    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[1] != xg.pad \
             or not ssq.is_contiguous():
-        raise KernelError(f"{what}: ssq must be contiguous float32 [shares, {share_rows(xg.shape[0])}]")
+        raise KernelError(f"{what}: ssq must be contiguous float32 [shares, {xg.pad}]")
 
 
 def skinny_after_chain(xg, ssq, eps: float, w, out_dtype=torch.bfloat16):
@@ -128,24 +163,29 @@ def skinny_after_chain(xg, ssq, eps: float, w, out_dtype=torch.bfloat16):
         raise KernelError(f"skinny_after_chain: output type {out_dtype}")
     out = torch.empty((M, N), dtype=out_dtype, device=w.device)
     check(library("gemm_bf16").gfa_skinny_after_chain_bf16(
-        ptr(xg), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w), ptr(out), _i(M), _i(N),
-        _i(K), _i(N), _i(0 if out_dtype == torch.bfloat16 else 1), _i(0), stream_handle()),
+        ptr(xg.data), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w), ptr(out), _i(M), _i(N),
+        _i(K), _i(N), _i(0 if out_dtype == torch.bfloat16 else 1), _i(0), _i(0), stream_handle()),
         "skinny_after_chain")
     return out
 
 
-def skinny_after_chain_gated(xg, ssq, eps: float, w13):
-    """silu(n W1^T) * (n W3^T) with n the normed rows given by their two halves."""
+def skinny_after_chain_gated(xg, ssq, eps: float, w13, chunked: bool = False):
+    """silu(n W1^T) * (n W3^T) with n the normed rows given by their two halves; ``chunked``:
+    as :class:`ChunkedRows`, for :func:`skinny_into_chain` to read."""
     _check_chain(xg, ssq, w13, "skinny_after_chain_gated")
     M, K = xg.shape
     if w13.shape[0] % 2:
         raise KernelError("skinny_after_chain_gated: w13 needs an even number of rows")
     I = w13.shape[0] // 2
-    out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
+    if chunked:
+        res = ChunkedRows(M, I, w13.device)
+        out = res.data
+    else:
+        res = out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
     check(library("gemm_bf16").gfa_skinny_after_chain_bf16(
-        ptr(xg), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I),
-        _i(K), _i(I), _i(3), _i(I), stream_handle()), "skinny_after_chain_gated")
-    return out
+        ptr(xg.data), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I),
+        _i(K), _i(I), _i(3), _i(I), _i(int(chunked)), stream_handle()), "skinny_after_chain_gated")
+    return res
 
 
 def wide_f32_out(x: torch.Tensor, w: torch.Tensor):
@@ -162,10 +202,12 @@ def qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages, n_
     """Fused q/k/v projection, rotation of interleaved pairs and the cache write in one
     kernel; returns q [M, H, hd].  ``x`` [M, K] bfloat16 holds normed rows (up to 64), or,
     with ``ssq`` and ``eps``, the two halves of a norm as :func:`skinny_into_chain` leaves
-    them (up to 16 rows).  k_pages None: nothing is stored."""
+    them (:class:`ChunkedRows`, up to 16 rows).  k_pages None: nothing is stored."""
     if ssq is not None:
         _check_chain(x, ssq, wqkv, "qkv_rope_store")
+        xdata = x.data
     else:
+        xdata = x
         _check_operands(x, wqkv, "qkv_rope_store")
         if wqkv.shape[1] % 8:
             raise KernelError("qkv_rope_store: the inner size must be a multiple of 8")
@@ -193,7 +235,7 @@ def qkv_rope_store(x, wqkv, freqs, tok_seq, tok_pos, table, k_pages, v_pages, n_
             raise KernelError("qkv_rope_store: pages have the wrong shape or dtype")
     q = torch.empty((M, n_heads, head_dim), dtype=torch.bfloat16, device=wqkv.device)
     check(library("gemm_bf16").gfa_qkv_rope_store_bf16(
-        ptr(x), ptr(ssq), _i(0 if ssq is None else ssq.shape[0]), ctypes.c_float(eps), ptr(wqkv),
+        ptr(xdata), ptr(ssq), _i(0 if ssq is None else ssq.shape[0]), ctypes.c_float(eps), ptr(wqkv),
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table),
         _i(table.shape[1]), _i(M), _i(K), _i(n_heads), _i(n_kv_heads), _i(head_dim),
         _i(rotary_dim), stream_handle()), "qkv_rope_store")

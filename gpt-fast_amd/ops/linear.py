@@ -57,7 +57,8 @@ def _fast():
 
 class HalfNormed:
     """Rows of an RMS norm in two halves, as the few-row product that completed the residual
-    stream left them: ``xg`` = bfloat16(residual * norm weight) [M, D] and ``ssq`` [shares, 16],
+    stream left them: ``xg`` = bfloat16(residual * norm weight) (``gemm_bf16.ChunkedRows``
+    of [M, D]) and ``ssq`` [shares, 4, 8 or 16],
     whose column sums are the rows' sums of squares (float32, from the float32 residual).
     The products of this module take it in place of x and apply the missing factor
     rsqrt(sum / D + eps) to their float32 result; a factor per row commutes with the product,
@@ -104,8 +105,7 @@ def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_n
     of this module) they are returned as a :class:`HalfNormed`; else None, and the caller runs
     the norm."""
     form = getattr(then_norm, "row_and_column_form", None)
-    if (form is not None and takes_halves and x.dtype == torch.bfloat16
-            and _fast().can_chain_norm(x.shape[0], w.shape[0], x.shape[1])):
+    if _chains(x.shape[0], x.dtype, w, then_norm, takes_halves):
         weight, eps = form()
         xg, ssq = _fast().skinny_into_chain(x, w, residual, weight)
         return HalfNormed(xg, ssq, eps)
@@ -117,6 +117,14 @@ def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_n
             return K.add_rmsnorm(residual, torch.matmul(x, w.t()), weight, eps)
     _linear_into(x, w, residual)
     return None
+
+
+def _chains(rows: int, dtype, w, then_norm, takes_halves: bool) -> bool:
+    """The few-row product with ``w`` that completes the residual stream also prepares
+    ``then_norm`` for a reader that takes it in halves."""
+    return (takes_halves and dtype == torch.bfloat16
+            and getattr(then_norm, "row_and_column_form", None) is not None
+            and _fast().can_chain_norm(rows, w.shape[0], w.shape[1]))
 
 
 def _wide():
@@ -151,6 +159,19 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
     if w13.shape[0] % 2 == 0 and _own_gate_is_faster(x.shape[0], w13.shape[0] // 2, x.shape[1], x.device):
         return _wide().product_gated(x, w13)
     return K.silu_mul(torch.matmul(x, w13.t()))
+
+
+def gated_into(x, w13: torch.Tensor, w2: torch.Tensor, residual: torch.Tensor, then_norm=None,
+               takes_halves: bool = False):
+    """residual += (silu(x W1^T) * (x W3^T)) W2^T: :func:`gated_linear`, then
+    :func:`linear_into` with its arguments and result.  Between two few-row kernels that take
+    and leave a norm in halves, the gate's result stays in the order the second one loads it
+    in (``gemm_bf16.ChunkedRows``)."""
+    if isinstance(x, HalfNormed) and _chains(x.shape[0], x.dtype, w2, then_norm, takes_halves):
+        h = _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13, chunked=True)
+    else:
+        h = gated_linear(x, w13)
+    return linear_into(h, w2, residual, then_norm, takes_halves)
 
 
 # ----------------------------------------------------------------------------- fused projection

@@ -31,8 +31,7 @@ class GatedFeedForward(Part):
     takes_prepared = 1
 
     def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
-        h = L.gated_linear(x, self.w13)
-        return L.linear_into(h, self.w2, residual, then_norm, takes_halves)
+        return L.gated_into(x, self.w13, self.w2, residual, then_norm, takes_halves)
 
 
 register_feed_forward("gated", GatedFeedForward)

@@ -581,7 +581,19 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
         assert float((got[m] - ref[m].cpu()).abs().max() / ref[m].abs().max()) < 1.5e-2
     # the two halves put together by hand are the norm's rows
     rs = torch.rsqrt(ssq.sum(0)[:M, None].double() / D + eps)
-    close(xg.double() * rs, n, 1e-2)
+    close(xg.to_rows().double() * rs, n, 1e-2)
+    # the gate's result left in the order the next product loads it in: the same values, and
+    # the same product from them
+    if I % 8 == 0:
+        h_rows = G.skinny_after_chain_gated(xg, ssq, eps, w)
+        h_chunked = G.skinny_after_chain_gated(xg, ssq, eps, w, chunked=True)
+        assert torch.equal(h_chunked.to_rows(), h_rows)
+        w2 = bf(torch.randn(D, I, device=DEV) * 0.2)
+        res_a, res_b = res0.clone(), res0.clone()
+        xg_a, ssq_a = G.skinny_into_chain(h_rows, w2, res_a, g)
+        xg_b, ssq_b = G.skinny_into_chain(h_chunked, w2, res_b, g)
+        assert torch.equal(res_a, res_b) and torch.equal(ssq_a, ssq_b)
+        assert torch.equal(xg_a.to_rows(), xg_b.to_rows())
 
 
 @pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
         bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
-        int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows) {
+        int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows, int out_pad) {
     constexpr int DT = DS * 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     static_assert(!SINGLE || RT == 1, "one token per sequence is one tile of rows");
@@ -318,6 +318,9 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         if (rpos[rt] < 0) continue;
         if (n_splits == 1) {
             const float inv = 1.f / lt[rt];
+            // out_pad (SINGLE only): the result is left chunked (common.h) for the product
+            // that reads it next; the row is the token, the column (head, dim)
+            const int tok = SINGLE ? seq : 0, col0 = SINGLE ? (int)(orow[rt] - (size_t)seq * H) * hd : 0;
             bf16_t* orow_p = out + orow[rt] * hd;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
@@ -326,7 +329,8 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
                     Frag w;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) w.e[j] = float_to_bf16(o[rt][dt][j] * inv);
-                    *(uint2*)(orow_p + d) = w.h[0];
+                    bf16_t* dst = (SINGLE && out_pad) ? out + chunked_elem(tok, col0 + d, out_pad) : orow_p + d;
+                    *(uint2*)dst = w.h[0];
                 }
             }
         } else {
@@ -694,8 +698,9 @@ extern "C" int gfa_attention_tiled_bf16(const void* q, const void* k_pages, cons
 __global__ __launch_bounds__(64) void attention_combine_kernel(const float* __restrict__ ws_o,
                                                                const float* __restrict__ ws_ml,
                                                                bf16_t* __restrict__ out, int hd,
-                                                               int n_splits, int total_rows) {
-    const int row = blockIdx.x, lane = threadIdx.x;
+                                                               int n_splits, int total_rows, int H,
+                                                               int out_pad) {
+    const int row = blockIdx.x, lane = threadIdx.x;      // row = token * H + head
     float ms = -INFINITY, ls = 0.f;
     if (lane < n_splits) {
         const float2 ml = *(const float2*)(ws_ml + ((size_t)lane * total_rows + row) * 2);
@@ -734,8 +739,11 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(const float* __re
             a1 += wj * v.y;
         }
         if (mine) {
-            out[(size_t)row * hd + d] = float_to_bf16(a0 * inv);
-            out[(size_t)row * hd + d + 1] = float_to_bf16(a1 * inv);
+            // out_pad: left chunked (common.h) for the product that reads it next
+            bf16_t* dst = out_pad ? out + chunked_elem(row / H, (row % H) * hd + d, out_pad)
+                                  : out + (size_t)row * hd + d;
+            dst[0] = float_to_bf16(a0 * inv);
+            dst[1] = float_to_bf16(a1 * inv);
         }
     }
 }
@@ -745,16 +753,16 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
                              const bf16_t* k, const bf16_t* v, const int* q_start,
                              const int* start_pos, const int* table, int table_stride, bf16_t* out,
                              float* ws_o, float* ws_ml, int H, int Hkv, int hd, float sl2, int window,
-                             int n_splits, int total_rows, bool single) {
+                             int n_splits, int total_rows, bool single, int out_pad) {
     const size_t shmem = nw > 1 ? (size_t)(nw - 1) * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
     if (rt == 1 && single)
-        attention_mfma_kernel<DS, 1, false, true><<<dim3(n_splits, grid.y, grid.z / n_splits), 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<DS, 1, false, true><<<dim3(n_splits, grid.y, grid.z / n_splits), 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, out_pad);
     else if (rt == 1)
-        attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
     else if (rt == 2)
-        attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
     else if (DS <= 4)
-        attention_mfma_kernel<(DS <= 4 ? DS : 4), 4, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows);
+        attention_mfma_kernel<(DS <= 4 ? DS : 4), 4, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
 }
 
 // q, out [n_tokens, H, hd]; the sequences' token runs are given by q_start [n_seqs + 1] and
@@ -763,16 +771,21 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
 // max_tiles = most waves any sequence needs per kv head.  With n_splits > 1, ws_o
 // [n_splits, n_tokens * H, hd] and ws_ml [n_splits, n_tokens * H, 2] hold the partials.
 // one_token_each: the caller vouches that q_start is 0, 1, 2, ... (every sequence one token).
+// out_chunked (with one_token_each, up to 16 tokens): out is left as chunked rows [n_tokens,
+// H * hd] (common.h: chunked_elem, pad = 4, 8 or 16) for the few-row product that reads it.
 extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void* v_pages,
                                   const int* q_start, const int* start_pos, const int* table,
                                   int table_stride, void* out, float* ws_o, float* ws_ml,
                                   int n_tokens, int n_seqs, int H, int Hkv, int hd, float scale,
                                   int window, int rt, int n_waves, int max_tiles, int n_splits,
-                                  int one_token_each, hipStream_t stream) {
+                                  int one_token_each, int out_chunked, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
     if (one_token_each && n_tokens != n_seqs) return (int)hipErrorInvalidValue;
     if ((long)table_stride * 2 * (n_splits + 1) >= (1L << 31)) return (int)hipErrorInvalidValue;
     const bool single = one_token_each && rt == 1 && max_tiles == 1 && H / Hkv <= 16;
+    // out_chunked: up to 16 tokens, one per sequence, (H * hd) % 8 == 0 (it is: hd % 16 == 0)
+    if (out_chunked && (!single || n_tokens > 16)) return (int)hipErrorInvalidValue;
+    const int out_pad = out_chunked ? (n_tokens <= 4 ? 4 : n_tokens <= 8 ? 8 : 16) : 0;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || n_splits > 64 || max_tiles < 1 ||
         !(scale > 0.f) ||                                 // the kernels take maxima before scaling
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||
@@ -786,12 +799,12 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     const bf16_t* kp = (const bf16_t*)k_pages;
     const bf16_t* vp = (const bf16_t*)v_pages;
     if (hd <= 64)
-        launch_attention<2>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
+        launch_attention<2>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single, out_pad);
     else if (hd <= 128)
-        launch_attention<4>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
+        launch_attention<4>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single, out_pad);
     else
-        launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single);
+        launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single, out_pad);
     if (n_splits > 1)
-        attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows);
+        attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows, H, out_pad);
     return GFA_LAUNCH_RESULT();
 }

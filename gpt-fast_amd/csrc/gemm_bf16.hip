@@ -30,14 +30,6 @@ __device__ __forceinline__ float dot8(const Pack8& a, const Pack8& b, float acc)
 
 __device__ __forceinline__ float silu(float a) { return a / (1.f + expf(-a)); }
 
-// Rows kept for a few-row product that reads them next ("chunked", pad = 4, 8 or 16 rows):
-// [columns / 8][pad][8] instead of [rows][columns], so that the sixteen lanes which load one
-// 16-byte chunk each of sixteen different rows read consecutive bytes (whole cache lines)
-// instead of sixteen lines.  Element (m, n) of such rows:
-__device__ __forceinline__ size_t chunked_elem(int m, int n, int pad) {
-    return ((size_t)(n >> 3) * pad + m) * 8 + (n & 7);
-}
-
 template <int MODE>
 __device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, float v, float gate_v,
                                              int out_pad = 0) {

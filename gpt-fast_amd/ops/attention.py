@@ -10,11 +10,14 @@ import torch
 from . import kernels as K
 
 
-def attention(q, k_pages, v_pages, batch, table, scale: float, window: int = 0):
-    """q [N, H, hd] of the step's tokens; returns [N, H, hd]."""
+def attention(q, k_pages, v_pages, batch, table, scale: float, window: int = 0,
+              for_product: bool = False):
+    """q [N, H, hd] of the step's tokens; returns [N, H, hd].  ``for_product``: the caller
+    only hands the result to a few-row product of ``ops.linear`` that takes
+    ``gemm_bf16.ChunkedRows`` ([N, H * hd]), and may get that instead."""
     if q.dtype == torch.bfloat16:
         from . import attention_bf16 as fast
-        y = fast.attention(q, k_pages, v_pages, batch, table, scale, window)
+        y = fast.attention(q, k_pages, v_pages, batch, table, scale, window, chunked=for_product)
         if y is not None:
             return y
     return K.attention_generic(q, k_pages, v_pages, batch.tok_seq, batch.tok_pos, table,

@@ -54,9 +54,11 @@ def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int)
     return rt, 1, (rows + 16 * rt - 1) // (16 * rt), 1
 
 
-def attention(q, k_pages, v_pages, batch, table, scale, window):
+def attention(q, k_pages, v_pages, batch, table, scale, window, chunked: bool = False):
     """The kernel's result [N, H, hd], or None if it does not take this shape (head sizes
-    that are no multiple of 16 or exceed 256 go to the plain kernel)."""
+    that are no multiple of 16 or exceed 256 go to the plain kernel).  ``chunked``: where the
+    step is one token for each of up to 16 sequences, the result [N, H * hd] is returned as
+    ``gemm_bf16.ChunkedRows``, the order in which the few-row product that follows loads it."""
     n, H, hd = q.shape
     G = k_pages.shape[1]
     if hd % 16 or hd > 256 or H % G:
@@ -80,7 +82,14 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
             "attention_tiled_bf16")
         return out
     rt, nw, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
-    out = torch.empty_like(q)
+    one_each = batch.max_q_len == 1 and n == batch.n_seqs
+    chunked = chunked and one_each and n <= 16 and tiles == 1
+    if chunked:
+        from .gemm_bf16 import ChunkedRows
+        res = ChunkedRows(n, H * hd, q.device)
+        out = res.data
+    else:
+        res = out = torch.empty_like(q)
     ws_o = ws_ml = None
     if splits > 1:
         ws_o = torch.empty((splits, n * H, hd), dtype=torch.float32, device=q.device)
@@ -89,7 +98,7 @@ def attention(q, k_pages, v_pages, batch, table, scale, window):
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(batch.q_start), ptr(batch.start_pos), ptr(table),
         _i(table.shape[1]), ptr(out), ptr(ws_o), ptr(ws_ml), _i(n), _i(batch.n_seqs), _i(H), _i(G),
         _i(hd), _f(scale), _i(window), _i(rt), _i(nw), _i(tiles), _i(splits),
-        _i(int(batch.max_q_len == 1 and n == batch.n_seqs)), stream_handle()),
+        _i(int(one_each)), _i(int(chunked)), stream_handle()),
         "attention_bf16")
-    return out
+    return res
 

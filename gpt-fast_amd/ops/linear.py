@@ -119,6 +119,12 @@ def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_n
     return None
 
 
+def takes_chunked_rows(rows: int, dtype, w, then_norm, takes_halves: bool) -> bool:
+    """:func:`linear_into` with these arguments runs the few-row kernel that also reads its x
+    as ``gemm_bf16.ChunkedRows``."""
+    return _chains(rows, dtype, w, then_norm, takes_halves)
+
+
 def _chains(rows: int, dtype, w, then_norm, takes_halves: bool) -> bool:
     """The few-row product with ``w`` that completes the residual stream also prepares
     ``then_norm`` for a reader that takes it in halves."""

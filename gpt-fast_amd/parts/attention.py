@@ -57,10 +57,13 @@ class Attention(Part):
             qkv = L.linear(x, self.wqkv)                                    # model.py:195
             q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
                                                s.head_dim)                  # model.py:201-207
+        # the output projection may take the heads' results in the order it loads them in
+        rows_for_wo = L.takes_chunked_rows(x.shape[0], q.dtype, self.wo, then_norm, takes_halves)
         y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
-                        self.scale, self.window)                            # model.py:209-211
-        return L.linear_into(y.view(x.shape[0], s.n_heads * s.head_dim), self.wo, residual,
-                             then_norm, takes_halves)                       # model.py:215, 162
+                        self.scale, self.window, for_product=rows_for_wo)   # model.py:209-211
+        if isinstance(y, torch.Tensor):
+            y = y.view(x.shape[0], s.n_heads * s.head_dim)
+        return L.linear_into(y, self.wo, residual, then_norm, takes_halves)  # model.py:215, 162
 
 
 register_mixer("attention", Attention)

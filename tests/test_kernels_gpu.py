@@ -338,8 +338,13 @@ def test_single_token_attention_in_a_batch(H, G, hd, window):
     """One new token for each sequence of a batch (the step that decoding repeats): lengths
     from one key to 4,100 in one launch - the last one's page row is longer than the 63
     entries a wave keeps in registers - on scattered pages with poisoned tails."""
+    _single_token_batch(H, G, hd, window, [1, 63, 64, 65, 200, 333, 4100, 2])
+    _single_token_batch(H, G, hd, window, [5, 333, 64, 129, 1])        # short: no context split
+
+
+def _single_token_batch(H, G, hd, window, lens):
     from gpt_fast_amd.ops import attention as A
-    lens = [1, 63, 64, 65, 200, 333, 4100, 2]
+    from gpt_fast_amd.ops.gemm_bf16 import ChunkedRows
     k_pages, v_pages, table, ks, vs = _paged(lens, G, hd, torch.bfloat16, seed=hd + H)
     g = torch.Generator().manual_seed(6)
     q = torch.randn(len(lens), H, hd, generator=g).to(torch.bfloat16)
@@ -360,6 +365,10 @@ def test_single_token_attention_in_a_batch(H, G, hd, window):
     for b, S in enumerate(lens):
         ref = _attention_ref(q[b].float(), ks[b].float(), vs[b].float(), S - 1, scale, window)
         close(out[b], ref, 1.5e-2)
+    # the same result in the order the output projection loads it in
+    rows = A.attention(q.to(DEV), k_pages, v_pages, batch, table, scale, window, for_product=True)
+    assert isinstance(rows, ChunkedRows) and rows.shape == (len(lens), H * hd)
+    assert torch.equal(rows.to_rows().cpu().view(len(lens), H, hd), out)
 
 
 @pytest.mark.parametrize("H,G,hd,window", [(8, 2, 128, 0), (4, 4, 64, 0), (6, 2, 96, 0), (8, 2, 128, 1000),

@@ -551,9 +551,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                                    fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7]))),
                              fmaxf(fmaxf(fmaxf(sv[8], sv[9]), fmaxf(sv[10], sv[11])),
                                    fmaxf(fmaxf(sv[12], sv[13]), fmaxf(sv[14], sv[15]))));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            mx *= scale_log2;                              // scale > 0: the order is kept
+            mx = max_over_lane_groups(mx) * scale_log2;    // scale > 0: the order is kept
             if (__builtin_amdgcn_ballot_w64(mx > m[rt] + TL_SLACK) != 0) {
                 // some row's maximum moved far: raise every row's reference and rescale
                 const float m_new = fmaxf(m[rt], mx);
@@ -609,8 +607,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        float lt = l[rt] + __shfl_xor(l[rt], 16, 64);
-        lt += __shfl_xor(lt, 32, 64);
+        const float lt = sum_over_lane_groups(l[rt]);
         if (rpos[rt] < 0) continue;
         const float inv = 1.f / lt;
         bf16_t* orow_p = out + orow[rt] * hd;

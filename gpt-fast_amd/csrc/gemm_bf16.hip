@@ -245,7 +245,7 @@ struct SkinnyExtra {
     int table_stride, H, Hkv, hd, rot;
     // A norm spread over two kernels (one tile of rows).  The kernel that completes the
     // residual stream (MODE 2) also writes xg_out = bfloat16(new residual * next_g) (chunked) and
-    // ssq_out [tiles, share_rows] (tiles of gfa_skinny_tile_rows(2, N) columns): each workgroup's share of its rows' sums of squares (float,
+    // ssq_out [gfa_skinny_workgroups(2, M, N), share_rows]: each workgroup's share of its rows' sums of squares (float,
     // from the float residual).  The next product takes xg as its x, adds the shares in a fixed
     // order (ssq_in [t_in, share_rows]) and scales its result by rsqrt(sum / K + eps): a factor per row
     // commutes with the product, so this is the RMS norm of model.py:236-241.
@@ -264,16 +264,22 @@ struct SkinnyExtra {
 // Rows per record of the sums-of-squares shares for M rows of x.
 extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-template <int CT, int MODE, int XP = 1, bool XF = false>
+// TILES = 2 (nine to sixteen rows of x, wide matrices, not the gate): a workgroup takes two
+// tiles of W's rows, one below the other, against the same fragments of x.  With sixteen
+// rows every workgroup reads as many bytes of x as of W; two tiles halve that, at half as
+// many workgroups, which pays where those still fill the chip.
+template <int CT, int MODE, int XP = 1, bool XF = false, int TILES = 1>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, int th, SkinnyExtra ex) {
-    constexpr int RT = (MODE == 3) ? 2 : 1;
+    static_assert(TILES == 1 || (TILES == 2 && CT == 1 && MODE != 3), "two tiles: one tile of x rows, no gate");
+    constexpr int RT = (MODE == 3) ? 2 : TILES;          // tiles of W's rows multiplied per x fragment
+    constexpr int NT = (MODE == 3) ? 1 : TILES;          // tiles of output columns per workgroup
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
-    // th (12..16) rows of W per workgroup: the host picks it so that the tiles divide evenly
+    // th (12..16) rows of W per tile: the host picks it so that the tiles divide evenly
     // over the compute units; operand rows th..15 repeat row th - 1 and are never stored
-    const int n0 = blockIdx.x * th;
+    const int n0 = blockIdx.x * th * NT;
     char* stage = smem + (size_t)wave * (RT * SM_TILE);
     const int lrow = lane >> 4, lchunk = lane & 15;      // loading: row lrow + 4 j, 16-byte chunk
     const int fi = lane & 15, fg = lane >> 4;            // multiplying: row / column fi, k group fg
@@ -295,9 +301,9 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int r = lrow + 4 * j;
-            int n = n0 + (r < th ? r : th - 1);
+            int n = n0 + (MODE == 3 ? 0 : rt * th) + (r < th ? r : th - 1);
             if (n >= N) n = N - 1;                       // clamped rows are computed, not stored
-            wsrc[rt][j] = w + (size_t)(n + rt * gate_rows) * K + lchunk * 8;
+            wsrc[rt][j] = w + (size_t)(n + (MODE == 3 ? rt * gate_rows : 0)) * K + lchunk * 8;
         }
     // two register sets: while piece t is multiplied, pieces t + 1 and t + 2 are in flight
     uint4 regs_a[RT][4], regs_b[RT][4];
@@ -405,34 +411,40 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     if (t_begin + 1 < t_end) load_piece(t_begin + 1, regs_b);
     // What the epilogue of wave 0 reads is requested now, behind the first pieces of W, so
     // that its latency (and the rotation's sine and cosine) passes while W streams.
-    float4 res_pre[CT], g_pre[CT];                       // MODE 2: the residual's old values, next norm's weights
-    bool res_ok[CT];
-    float rot_cs[2] = {1.f, 1.f}, rot_sn[2] = {0.f, 0.f};   // MODE 4, one tile of rows
-    int rot_pos = 0, rot_page = 0;
+    float4 res_pre[NT][CT], g_pre[NT][CT];               // MODE 2: the residual's old values, next norm's weights
+    bool res_ok[NT][CT];
+    float rot_cs[NT][2], rot_sn[NT][2];                  // MODE 4, one tile of rows
+    int rot_pos = 0, rot_page = 0;                       // the token's page serves both tiles
     constexpr bool ROT_EARLY = MODE == 4 && CT == 1;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        res_ok[ct] = false;
-        if (MODE == 2 && wave == 0) {
-            const int m = ct * 16 + fi, n = n0 + fg * 4;
-            res_ok[ct] = m < M && n + 3 < N && (ldo & 3) == 0 && fg * 4 + 3 < th;
-            if (res_ok[ct]) {
-                res_pre[ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
-                if (ex.xg_out) g_pre[ct] = *(const float4*)(ex.next_g + n);
+    for (int ot = 0; ot < NT; ++ot) {
+        const int nb = n0 + ot * th;                     // first column of this output tile
+        rot_cs[ot][0] = rot_cs[ot][1] = 1.f;
+        rot_sn[ot][0] = rot_sn[ot][1] = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            res_ok[ot][ct] = false;
+            if (MODE == 2 && wave == 0) {
+                const int m = ct * 16 + fi, n = nb + fg * 4;
+                res_ok[ot][ct] = m < M && n + 3 < N && (ldo & 3) == 0 && fg * 4 + 3 < th;
+                if (res_ok[ot][ct]) {
+                    res_pre[ot][ct] = *(const float4*)((const float*)out + (size_t)m * ldo + n);
+                    if (ex.xg_out) g_pre[ot][ct] = *(const float4*)(ex.next_g + n);
+                }
             }
         }
-    }
-    if (ROT_EARLY && wave == 0 && fi < M && n0 + fg * 4 < N && fg * 4 < th) {
-        const int n = n0 + fg * 4;
-        const int head = n / ex.hd, d = n - head * ex.hd;
-        rot_pos = ex.tok_pos[fi];
-        if (head >= ex.H && ex.k_pages)
-            rot_page = ex.table[(size_t)ex.tok_seq[fi] * ex.table_stride + rot_pos / GFA_PAGE];
-        if (head < ex.H + ex.Hkv) {
+        if (ROT_EARLY && wave == 0 && fi < M && nb + fg * 4 < N && fg * 4 < th) {
+            const int n = nb + fg * 4;
+            const int head = n / ex.hd, d = n - head * ex.hd;
+            rot_pos = ex.tok_pos[fi];
+            if (head >= ex.H && ex.k_pages)
+                rot_page = ex.table[(size_t)ex.tok_seq[fi] * ex.table_stride + rot_pos / GFA_PAGE];
+            if (head < ex.H + ex.Hkv) {
 #pragma unroll
-            for (int pr = 0; pr < 2; ++pr)
-                if (d + 2 * pr < ex.rot)
-                    sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[pr], &rot_cs[pr]);
+                for (int pr = 0; pr < 2; ++pr)
+                    if (d + 2 * pr < ex.rot)
+                        sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[ot][pr], &rot_cs[ot][pr]);
+            }
         }
     }
     // second half of a two-kernel norm.  A share record holds R = share_rows rows side by
@@ -513,28 +525,34 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         }
     }
     float part_ssq = 0.f;                                // MODE 2 with xg_out: this lane's r^2
+    if (chained) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const int m = ct * 16 + fi;
-        if (m >= M) continue;
-        if (chained) {
+        for (int ct = 0; ct < CT; ++ct) {
             const float rs = rsqrtf(ssq[ct] / (float)K + ex.eps);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) acc[rt][ct] *= rs;
         }
+    }
+#pragma unroll
+    for (int ot = 0; ot < NT; ++ot)                      // the workgroup's tiles of output columns
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int m = ct * 16 + fi;
+        const int nb = n0 + ot * th;                     // first column of this tile
+        if (m >= M) continue;
         if (MODE == 4) {
-            // columns n0 + 4 fg .. +3 of token m: two rotary pairs of one head
-            const int n = n0 + fg * 4;
+            // columns nb + 4 fg .. +3 of token m: two rotary pairs of one head
+            const int n = nb + fg * 4;
             if (n >= N || fg * 4 >= th) continue;        // th is a multiple of 4 here
             const int hd = ex.hd, head = n / hd, d = n - head * hd;
             const int pos = ROT_EARLY ? rot_pos : ex.tok_pos[m];
-            float v[4] = {acc[0][ct][0], acc[0][ct][1], acc[0][ct][2], acc[0][ct][3]};
+            float v[4] = {acc[ot][ct][0], acc[ot][ct][1], acc[ot][ct][2], acc[ot][ct][3]};
             if (head < ex.H + ex.Hkv) {
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     const int dd = d + 2 * pr;
                     if (dd < ex.rot) {
-                        float sn = rot_sn[pr], cs = rot_cs[pr];
+                        float sn = rot_sn[ot][pr], cs = rot_cs[ot][pr];
                         if (!ROT_EARLY) sincosf((float)pos * ex.freqs[dd >> 1], &sn, &cs);
                         const float a = v[2 * pr], bb = v[2 * pr + 1];
                         v[2 * pr] = a * cs - bb * sn;
@@ -562,30 +580,30 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                         ex.v_pages[value_elem(page, g, d + j, off, ex.Hkv, hd)] = e[j];
                 }
             }
-        } else if (MODE == 2 && res_ok[ct]) {
-            float4 r = res_pre[ct];                      // the same sums as skinny_store<2>
-            r.x += acc[0][ct][0];
-            r.y += acc[0][ct][1];
-            r.z += acc[0][ct][2];
-            r.w += acc[0][ct][3];
-            *(float4*)((float*)out + (size_t)m * ldo + n0 + fg * 4) = r;
+        } else if (MODE == 2 && res_ok[ot][ct]) {
+            float4 r = res_pre[ot][ct];                  // the same sums as skinny_store<2>
+            r.x += acc[ot][ct][0];
+            r.y += acc[ot][ct][1];
+            r.z += acc[ot][ct][2];
+            r.w += acc[ot][ct][3];
+            *(float4*)((float*)out + (size_t)m * ldo + nb + fg * 4) = r;
             if (ex.xg_out) {                             // first half of the next norm; N == ldo
-                const float4 g = g_pre[ct];
+                const float4 g = g_pre[ot][ct];
                 Frag8 pk;
                 bf16_t* e = (bf16_t*)&pk.u;
                 e[0] = float_to_bf16(r.x * g.x);
                 e[1] = float_to_bf16(r.y * g.y);
                 e[2] = float_to_bf16(r.z * g.z);
                 e[3] = float_to_bf16(r.w * g.w);
-                *(uint2*)(ex.xg_out + chunked_elem(m, n0 + fg * 4, ex.share_rows)) = make_uint2(pk.u.x, pk.u.y);
-                part_ssq = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
+                *(uint2*)(ex.xg_out + chunked_elem(m, nb + fg * 4, ex.share_rows)) = make_uint2(pk.u.x, pk.u.y);
+                part_ssq += fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
             }
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int n = n0 + fg * 4 + j;
+                const int n = nb + fg * 4 + j;
                 if (n < N && fg * 4 + j < th)
-                    skinny_store<MODE>(out, ldo, m, n, acc[0][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f, ex.out_pad);
+                    skinny_store<MODE>(out, ldo, m, n, acc[ot][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f, ex.out_pad);
             }
         }
     }
@@ -614,14 +632,14 @@ static int compute_units() {
 // much as the others; with 12 rows they are 512, two each.  The taller tile on a tie.  Not
 // below 12: every tile reads all of x, so lower tiles cost in x what they save in W (10240
 // columns at 8 rows, 1280 tiles for 640, measured 54 against 41 us at 16 rows of x).
-static int pick_tile_rows(int N, int step) {
+static int pick_tile_rows(int N, int step, int nt = 1) {
     const int cus = compute_units();
-    const long tiles16 = (N + 15) / 16;
+    const long tiles16 = (N + 16 * nt - 1) / (16 * nt);
     const long cost16 = ((tiles16 + cus - 1) / cus) * 16;
     int best = 16;
     long best_cost = cost16;
     for (int th = 16 - step; th >= 12; th -= step) {
-        const long tiles = (N + th - 1) / th;
+        const long tiles = (N + th * nt - 1) / (th * nt);
         const long cost = ((tiles + cus - 1) / cus) * th;
         if (cost < best_cost) {
             best = th;
@@ -633,21 +651,36 @@ static int pick_tile_rows(int N, int step) {
     return best_cost * 20 <= cost16 * 19 ? best : 16;
 }
 
-// Tile height the launcher below uses for this mode and width (the two-kernel norm's
-// shares are one record per tile, so its callers size their buffers by it).
-extern "C" int gfa_skinny_tile_rows(int mode, int N) {
-    return pick_tile_rows(N, (mode == 2 || mode == 4) ? 4 : 1);
+// Tiles of W's rows per workgroup: two for nine to sixteen rows of x where the workgroups
+// still fill the chip (measured on 256 compute units: a gain from 8192 rows of W on - 70B's
+// second feed-forward product 89 -> 81 us at sixteen rows of x -, a loss of a third with 4096).
+static int tiles_per_workgroup(int mode, int M, int N) {
+    return (mode != 3 && M > 8 && M <= 16 && N >= 32 * compute_units()) ? 2 : 1;
+}
+
+// Tile height the launcher below uses for this mode, these rows of x and this width.
+static int tile_rows(int mode, int M, int N) {
+    return pick_tile_rows(N, (mode == 2 || mode == 4) ? 4 : 1, tiles_per_workgroup(mode, M, N));
+}
+
+// Workgroups the launcher below starts for this mode, M <= 16 rows of x and N columns (the
+// two-kernel norm's shares are one record per workgroup of mode 2, so its callers size
+// their buffers by it).
+extern "C" int gfa_skinny_workgroups(int mode, int M, int N) {
+    const int per = tile_rows(mode, M, N) * tiles_per_workgroup(mode, M, N);
+    return (N + per - 1) / per;
 }
 
 template <int MODE>
 static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
                               int ldo, int gate_rows, const SkinnyExtra& ex, hipStream_t stream) {
-    constexpr int RT = (MODE == 3) ? 2 : 1;
     const int ct = (M + 15) / 16;
     // the epilogues that add into the residual stream or rotate pairs work on groups of
     // four columns: their tiles are 12 or 16 rows high
-    const int th = ct == 1 ? gfa_skinny_tile_rows(MODE, N) : 16;
-    const int tiles = (N + th - 1) / th;
+    const int nt = ct == 1 ? tiles_per_workgroup(MODE, M, N) : 1;
+    const int th = ct == 1 ? tile_rows(MODE, M, N) : 16;
+    const int tiles = (N + th * nt - 1) / (th * nt);     // workgroups
+    const int RT = (MODE == 3) ? 2 : nt;                 // tiles of W staged per wave
     const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
     int nw = 1;                                          // waves per tile: aim at >= 2048 waves,
     const int nw_max = (MODE == 3) ? 4 : 8;
@@ -668,25 +701,26 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         exl.share_off = (int)shmem;
         shmem += (size_t)nw * 16 * 64 * sizeof(float);
     }
-#define GFA_LAUNCH_MFMA(CTV, XPV, XFV)                                                                 \
+#define GFA_LAUNCH_MFMA(CTV, XPV, XFV, NTV)                                                            \
     do {                                                                                          \
         static bool raised = false;                                                               \
         if (!raised) {                                                                            \
-            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV, XFV>,                  \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);           \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV>,             \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);          \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, XPV, XFV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, th, exl); \
+        skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, th, exl); \
     } while (0)
     switch (ct) {
         case 1:                                          // columns of the x operand that stand
-            if (M <= 4) GFA_LAUNCH_MFMA(1, 4, false);      // for no row carry later steps of k
-            else if (M <= 8) GFA_LAUNCH_MFMA(1, 2, false);
-            else GFA_LAUNCH_MFMA(1, 1, true);
+            if (M <= 4) GFA_LAUNCH_MFMA(1, 4, false, 1);   // for no row carry later steps of k
+            else if (M <= 8) GFA_LAUNCH_MFMA(1, 2, false, 1);
+            else if (nt == 2) GFA_LAUNCH_MFMA(1, 1, true, (MODE == 3 ? 1 : 2));
+            else GFA_LAUNCH_MFMA(1, 1, true, 1);
             break;
-        case 2: GFA_LAUNCH_MFMA(2, 1, false); break;
-        case 3: GFA_LAUNCH_MFMA(3, 1, false); break;
-        default: GFA_LAUNCH_MFMA(4, 1, false); break;
+        case 2: GFA_LAUNCH_MFMA(2, 1, false, 1); break;
+        case 3: GFA_LAUNCH_MFMA(3, 1, false, 1); break;
+        default: GFA_LAUNCH_MFMA(4, 1, false, 1); break;
     }
 #undef GFA_LAUNCH_MFMA
     return GFA_LAUNCH_RESULT();
@@ -748,7 +782,7 @@ extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t
 // residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
 // xg_out = bfloat16(new residual * next_g), kept chunked ([N / 8][share_rows][8], see
 // chunked_elem), ssq_out [tiles, share_rows] = the workgroups' shares of the rows' sums of
-// squares, tiles = N / gfa_skinny_tile_rows(2, N) rounded up; share_rows = gfa_share_rows(M).
+// squares, tiles = gfa_skinny_workgroups(2, M, N); share_rows = gfa_share_rows(M).
 // N a multiple of 8.  x_chunked: x is kept chunked too (pad gfa_share_rows(M)), as the gate
 // of gfa_skinny_after_chain_bf16 leaves its result on request.
 extern "C" int gfa_skinny_into_chain_bf16(const void* x, int x_chunked, const void* w,

@@ -119,7 +119,7 @@ def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:
 def skinny_into_chain(x, w: torch.Tensor, residual: torch.Tensor, next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
     ``xg`` = bfloat16(new residual * next_g) as :class:`ChunkedRows` and ``ssq`` float32
-    [tiles, R]: per workgroup (a tile of 12 to 16 columns) its share of each row's sum of
+    [workgroups, R]: per workgroup (one or two tiles of 12 to 16 columns) its share of each row's sum of
     squares, R = 4, 8 or 16 rows per record (the least that holds M).  Up to 16 rows; x a
     tensor [M, K] or :class:`ChunkedRows` (the gate's result, left so on request)."""
     chunked = isinstance(x, ChunkedRows)
@@ -134,8 +134,8 @@ def skinny_into_chain(x, w: torch.Tensor, residual: torch.Tensor, next_g: torch.
     if not can_chain_norm(M, N, K):
         raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
     xg = ChunkedRows(M, N, w.device)
-    th = library("gemm_bf16").gfa_skinny_tile_rows(_i(2), _i(N))     # one record per tile of columns
-    ssq = torch.empty(((N + th - 1) // th, share_rows(M)), dtype=torch.float32, device=w.device)
+    records = library("gemm_bf16").gfa_skinny_workgroups(_i(2), _i(M), _i(N))   # one per workgroup
+    ssq = torch.empty((records, share_rows(M)), dtype=torch.float32, device=w.device)
     check(library("gemm_bf16").gfa_skinny_into_chain_bf16(
         ptr(x.data if chunked else x), _i(int(chunked)), ptr(w), ptr(residual), _i(M), _i(N), _i(K),
         ptr(next_g), ptr(xg.data), ptr(ssq), stream_handle()), "skinny_into_chain")

@@ -605,6 +605,56 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
         assert torch.equal(xg_a.to_rows(), xg_b.to_rows())
 
 
+@pytest.mark.parametrize("M", [9, 12, 16])
+def test_wide_matrices_at_nine_to_sixteen_rows(M):
+    """From 8,192 rows of W on, a workgroup of the few-row kernel takes two tiles of W against
+    the same fragments of x (nine to sixteen rows of x): every epilogue on such a shape, the
+    last workgroup with a second tile that is partly or wholly beyond the matrix."""
+    from gpt_fast_amd.ops import gemm_bf16 as G
+    torch.manual_seed(M)
+    K_ = 264
+    for N in (8192, 8200, 8216):
+        x = bf(torch.randn(M, K_, device=DEV))
+        w = bf(torch.randn(N, K_, device=DEV) * 0.1)
+        ref = x.double() @ w.double().T
+        close(G.skinny(x, w, out_dtype=torch.float32), ref, 1e-5)
+        close(G.skinny(x, w), ref, 1e-2)
+        res0 = torch.randn(M, N, device=DEV)
+        res = res0.clone()
+        G.skinny(x, w, residual=res)
+        close(res, res0.double() + ref, 1e-5)
+        # the norm in two halves: produced on the wide shape, consumed by a wide shape
+        g = 1 + 0.1 * torch.randn(N, device=DEV)
+        res = res0.clone()
+        xg, ssq = G.skinny_into_chain(x, w, res, g)
+        new = res0.double() + ref
+        close(res, new, 1e-5)
+        close(ssq.sum(0)[:M], (new ** 2).sum(1), 1e-5)
+        eps = 1e-5
+        n = new * torch.rsqrt((new ** 2).mean(-1, keepdim=True) + eps) * g.double()
+        close(xg.to_rows().double() * torch.rsqrt(ssq.sum(0)[:M, None].double() / N + eps), n, 1e-2)
+        w2 = bf(torch.randn(8192 + 16, N, device=DEV) * 0.02)
+        close(G.skinny_after_chain(xg, ssq, eps, w2, out_dtype=torch.float32), n @ w2.double().T, 1e-2)
+    # projection, rotation and cache write: 64 heads of 128 are 8,192 rows of W
+    H, G_, hd = 48, 8, 128
+    pos = [3, 64, 200][:1] * M
+    tok_seq = torch.arange(M, dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor([5 + 7 * i for i in range(M)], dtype=torch.int32, device=DEV)
+    table = torch.arange(M * 4, dtype=torch.int32, device=DEV).view(M, 4)
+    freqs = (1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))).to(DEV)
+    xn = bf(torch.randn(M, K_, device=DEV))
+    wq = bf(torch.randn((H + 2 * G_) * hd, K_, device=DEV) * 0.1)
+    kp = torch.zeros(M * 4, G_, 64, hd, device=DEV, dtype=torch.bfloat16)
+    vp = torch.zeros(M * 4, G_, hd, 64, device=DEV, dtype=torch.bfloat16)
+    q = G.qkv_rope_store(xn, wq, freqs, tok_seq, tok_pos, table, kp, vp, H, G_, hd, hd)
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    q2 = K().rope_cache_write(G.skinny(xn, wq), freqs, tok_seq, tok_pos, table, kp2, vp2, H, G_, hd, hd, 0)
+    close(q, q2, 1e-2)
+    close(kp, kp2, 1e-2)
+    assert torch.equal(vp, vp2)
+    assert torch.equal(kp == 0, kp2 == 0) and torch.equal(vp == 0, vp2 == 0)
+
+
 @pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])
 def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     from gpt_fast_amd.ops import gemm_bf16 as G

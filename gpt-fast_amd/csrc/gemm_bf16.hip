@@ -652,10 +652,11 @@ static int pick_tile_rows(int N, int step, int nt = 1) {
 }
 
 // Tiles of W's rows per workgroup: two for nine to sixteen rows of x where the workgroups
-// still fill the chip (measured on 256 compute units: a gain from 8192 rows of W on - 70B's
-// second feed-forward product 89 -> 81 us at sixteen rows of x -, a loss of a third with 4096).
+// still fill three quarters of the chip (measured on 256 compute units at sixteen rows of x:
+// 8192 x 28672 89 -> 79 us, 8192 x 8192 30.6 -> 26.5, 6144 x 4096 14.2 -> 12.8; with 4096 rows
+// of W, 128 workgroups, a loss of a fifth).
 static int tiles_per_workgroup(int mode, int M, int N) {
-    return (mode != 3 && M > 8 && M <= 16 && N >= 32 * compute_units()) ? 2 : 1;
+    return (mode != 3 && M > 8 && M <= 16 && N >= 24 * compute_units()) ? 2 : 1;
 }
 
 // Tile height the launcher below uses for this mode, these rows of x and this width.

@@ -768,8 +768,8 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
 // max_tiles = most waves any sequence needs per kv head.  With n_splits > 1, ws_o
 // [n_splits, n_tokens * H, hd] and ws_ml [n_splits, n_tokens * H, 2] hold the partials.
 // one_token_each: the caller vouches that q_start is 0, 1, 2, ... (every sequence one token).
-// out_chunked (with one_token_each, up to 16 tokens): out is left as chunked rows [n_tokens,
-// H * hd] (common.h: chunked_elem, pad = 4, 8 or 16) for the few-row product that reads it.
+// out_chunked (with one_token_each, up to 64 tokens): out is left as chunked rows [n_tokens,
+// H * hd] (common.h: chunked_elem) for the few-row product that reads it.
 extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void* v_pages,
                                   const int* q_start, const int* start_pos, const int* table,
                                   int table_stride, void* out, float* ws_o, float* ws_ml,
@@ -780,9 +780,10 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
     if (one_token_each && n_tokens != n_seqs) return (int)hipErrorInvalidValue;
     if ((long)table_stride * 2 * (n_splits + 1) >= (1L << 31)) return (int)hipErrorInvalidValue;
     const bool single = one_token_each && rt == 1 && max_tiles == 1 && H / Hkv <= 16;
-    // out_chunked: up to 16 tokens, one per sequence, (H * hd) % 8 == 0 (it is: hd % 16 == 0)
-    if (out_chunked && (!single || n_tokens > 16)) return (int)hipErrorInvalidValue;
-    const int out_pad = out_chunked ? (n_tokens <= 4 ? 4 : n_tokens <= 8 ? 8 : 16) : 0;
+    // out_chunked: up to 64 tokens, one per sequence, (H * hd) % 8 == 0 (it is: hd % 16 == 0)
+    if (out_chunked && (!single || n_tokens > 64)) return (int)hipErrorInvalidValue;
+    const int out_pad = !out_chunked ? 0 : n_tokens <= 4 ? 4 : n_tokens <= 8 ? 8 : n_tokens <= 16 ? 16
+                                         : n_tokens <= 32 ? 32 : 64;
     if (hd % 16 != 0 || hd > 256 || H % Hkv != 0 || n_splits < 1 || n_splits > 64 || max_tiles < 1 ||
         !(scale > 0.f) ||                                 // the kernels take maxima before scaling
         (rt != 1 && rt != 2 && rt != 4) || (rt == 4 && hd > 128) ||

@@ -122,8 +122,8 @@ __device__ __forceinline__ size_t value_elem(int page, int kv_head, int d, int k
     return cache_region(page, kv_head, n_kv_heads, head_dim) + value_offset(d, key, head_dim);
 }
 
-// Rows kept for a few-row product that reads them next ("chunked", pad = 4, 8 or 16 rows, the
-// least that holds them): [columns / 8][pad][8] instead of [rows][columns], so that the
+// Rows kept for a few-row product that reads them next ("chunked", pad = 4, 8, 16, 32 or 64
+// rows, the least that holds them): [columns / 8][pad][8] instead of [rows][columns], so that the
 // sixteen lanes which load one 16-byte chunk each of sixteen different rows read consecutive
 // bytes (whole cache lines) instead of sixteen lines.  Element (m, n) of such rows:
 __device__ __forceinline__ size_t chunked_elem(int m, int n, int pad) {

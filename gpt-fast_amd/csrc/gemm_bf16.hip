@@ -223,6 +223,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 #define SM_SUBK 128
 #define SM_PITCH (SM_SUBK * 2 + 16)          // bytes per staged row: 256 + pad against conflicts
 #define SM_TILE (16 * SM_PITCH)
+#define GFA_MAX_SHARE_COPIES 64
 
 union Frag8 {
     uint4 u;
@@ -255,16 +256,17 @@ struct SkinnyExtra {
     const float* ssq_in;
     int t_in;
     int share_off;            // byte offset in LDS of the waves' pieces for the shares
-    int share_rows;           // rows per share record: 4, 8 or 16 (the least that holds M)
+    int share_copies;         // copy instructions per wave that bring the shares into LDS
+    int share_rows;           // rows per share record: 4, 8, 16, 32 or 64 (the least that holds M)
     // chunked rows (see chunked_elem): x is read so if x_pad > 0; the gate's output (MODE 3)
     // is written so if out_pad > 0; xg_out always is, with share_rows as its pad
     int x_pad, out_pad;
 };
 
 // Rows per record of the sums-of-squares shares for M rows of x.
-extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
+extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : M <= 16 ? 16 : M <= 32 ? 32 : 64; }
 
-// TILES = 2 (nine to sixteen rows of x, wide matrices, not the gate): a workgroup takes two
+// TILES = 2 (nine to 48 rows of x, wide matrices, not the gate): a workgroup takes two
 // tiles of W's rows, one below the other, against the same fragments of x.  With sixteen
 // rows every workgroup reads as many bytes of x as of W; two tiles halve that, at half as
 // many workgroups, which pays where those still fill the chip.
@@ -272,7 +274,7 @@ template <int CT, int MODE, int XP = 1, bool XF = false, int TILES = 1>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, int th, SkinnyExtra ex) {
-    static_assert(TILES == 1 || (TILES == 2 && CT == 1 && MODE != 3), "two tiles: one tile of x rows, no gate");
+    static_assert(TILES == 1 || (TILES == 2 && CT <= 3 && MODE != 3), "two tiles: up to 48 rows of x, no gate");
     constexpr int RT = (MODE == 3) ? 2 : TILES;          // tiles of W's rows multiplied per x fragment
     constexpr int NT = (MODE == 3) ? 1 : TILES;          // tiles of output columns per workgroup
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -413,16 +415,18 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     // that its latency (and the rotation's sine and cosine) passes while W streams.
     float4 res_pre[NT][CT], g_pre[NT][CT];               // MODE 2: the residual's old values, next norm's weights
     bool res_ok[NT][CT];
-    float rot_cs[NT][2], rot_sn[NT][2];                  // MODE 4, one tile of rows
-    int rot_pos = 0, rot_page = 0;                       // the token's page serves both tiles
-    constexpr bool ROT_EARLY = MODE == 4 && CT == 1;
+    float rot_cs[NT][CT][2], rot_sn[NT][CT][2];          // MODE 4: cosine and sine of this lane's two pairs
+    int rot_pos[CT], rot_page[CT];                       // a token's page serves all tiles of columns
+    constexpr bool ROT_EARLY = MODE == 4;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) rot_pos[ct] = rot_page[ct] = 0;
 #pragma unroll
     for (int ot = 0; ot < NT; ++ot) {
         const int nb = n0 + ot * th;                     // first column of this output tile
-        rot_cs[ot][0] = rot_cs[ot][1] = 1.f;
-        rot_sn[ot][0] = rot_sn[ot][1] = 0.f;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
+            rot_cs[ot][ct][0] = rot_cs[ot][ct][1] = 1.f;
+            rot_sn[ot][ct][0] = rot_sn[ot][ct][1] = 0.f;
             res_ok[ot][ct] = false;
             if (MODE == 2 && wave == 0) {
                 const int m = ct * 16 + fi, n = nb + fg * 4;
@@ -433,17 +437,22 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                 }
             }
         }
-        if (ROT_EARLY && wave == 0 && fi < M && nb + fg * 4 < N && fg * 4 < th) {
-            const int n = nb + fg * 4;
-            const int head = n / ex.hd, d = n - head * ex.hd;
-            rot_pos = ex.tok_pos[fi];
-            if (head >= ex.H && ex.k_pages)
-                rot_page = ex.table[(size_t)ex.tok_seq[fi] * ex.table_stride + rot_pos / GFA_PAGE];
-            if (head < ex.H + ex.Hkv) {
 #pragma unroll
-                for (int pr = 0; pr < 2; ++pr)
-                    if (d + 2 * pr < ex.rot)
-                        sincosf((float)rot_pos * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[ot][pr], &rot_cs[ot][pr]);
+        for (int ct = 0; ct < CT; ++ct) {
+            const int m = ct * 16 + fi;
+            if (ROT_EARLY && wave == 0 && m < M && nb + fg * 4 < N && fg * 4 < th) {
+                const int n = nb + fg * 4;
+                const int head = n / ex.hd, d = n - head * ex.hd;
+                rot_pos[ct] = ex.tok_pos[m];
+                if (head >= ex.H && ex.k_pages)
+                    rot_page[ct] = ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + rot_pos[ct] / GFA_PAGE];
+                if (head < ex.H + ex.Hkv) {
+#pragma unroll
+                    for (int pr = 0; pr < 2; ++pr)
+                        if (d + 2 * pr < ex.rot)
+                            sincosf((float)rot_pos[ct] * ex.freqs[(d + 2 * pr) >> 1], &rot_sn[ot][ct][pr],
+                                    &rot_cs[ot][ct][pr]);
+                }
             }
         }
     }
@@ -453,12 +462,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     // wave-private piece of LDS - no register waits for them, so nothing below is held up -
     // and are added after the product.  Every workgroup reads all shares, so their bytes
     // count: hence the narrow records for few rows.
-    constexpr int SHARES = 16;
-    const bool chained = CT == 1 && ex.ssq_in != nullptr;
+    // copy instructions per wave: as many as bring in all records (the launcher sizes the LDS
+    // piece by it), at most GFA_MAX_SHARE_COPIES; records beyond are read at the end, one
+    // round trip after the other
+    const int SHARES = ex.share_copies;
+    const bool chained = ex.ssq_in != nullptr;
     float* share_lds = (float*)(smem + ex.share_off) + wave * (SHARES * 64);
     const int R = ex.share_rows, per_copy = R ? 64 / R : 4;
     if (chained) {
-#pragma unroll
         for (int j = 0; j < SHARES; ++j) {
             const int first = per_copy * (wave + NW * j);
             if (first < ex.t_in) {                         // wave-uniform
@@ -485,7 +496,6 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     if (chained) {                                       // fixed order: lane, lanes of a row, waves
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the copies into LDS have landed
         float pre_ssq = 0.f;
-#pragma unroll
         for (int j = 0; j < SHARES; ++j) {
             const int rec = per_copy * (wave + NW * j) + lane / R;
             if (rec < ex.t_in) pre_ssq += share_lds[j * 64 + lane];
@@ -497,7 +507,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             const float other = __shfl_xor(pre_ssq, step, GFA_WAVE);
             pre_ssq = (lane & step) ? other + pre_ssq : pre_ssq + other;
         }
-        ssq[0] = pre_ssq;                                // this wave's part of the row's sum
+        // now every lane l holds the wave's part of the sum of row l % R; row 16 ct + fi is this
+        // lane's in tile ct
+        if (CT == 1) {
+            ssq[0] = pre_ssq;                            // R <= 16: row fi is lane fi's, whatever fg
+        } else {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) ssq[ct] = __shfl(pre_ssq, ct * 16 + fi, GFA_WAVE);
+        }
     }
     if (NW > 1) {
         __syncthreads();                                 // staging is done; reuse it for the sums
@@ -524,7 +541,9 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             }
         }
     }
-    float part_ssq = 0.f;                                // MODE 2 with xg_out: this lane's r^2
+    float part_ssq[CT];                                  // MODE 2 with xg_out: this lane's r^2 per tile of rows
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) part_ssq[ct] = 0.f;
     if (chained) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -545,15 +564,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             const int n = nb + fg * 4;
             if (n >= N || fg * 4 >= th) continue;        // th is a multiple of 4 here
             const int hd = ex.hd, head = n / hd, d = n - head * hd;
-            const int pos = ROT_EARLY ? rot_pos : ex.tok_pos[m];
+            const int pos = rot_pos[ct];
             float v[4] = {acc[ot][ct][0], acc[ot][ct][1], acc[ot][ct][2], acc[ot][ct][3]};
             if (head < ex.H + ex.Hkv) {
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     const int dd = d + 2 * pr;
                     if (dd < ex.rot) {
-                        float sn = rot_sn[ot][pr], cs = rot_cs[ot][pr];
-                        if (!ROT_EARLY) sincosf((float)pos * ex.freqs[dd >> 1], &sn, &cs);
+                        const float sn = rot_sn[ot][ct][pr], cs = rot_cs[ot][ct][pr];
                         const float a = v[2 * pr], bb = v[2 * pr + 1];
                         v[2 * pr] = a * cs - bb * sn;
                         v[2 * pr + 1] = bb * cs + a * sn;
@@ -567,8 +585,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             if (head < ex.H) {
                 *(uint2*)(ex.q_out + ((size_t)m * ex.H + head) * hd + d) = make_uint2(pk.u.x, pk.u.y);
             } else if (ex.k_pages) {
-                const int page = ROT_EARLY ? rot_page
-                    : ex.table[(size_t)ex.tok_seq[m] * ex.table_stride + pos / GFA_PAGE];
+                const int page = rot_page[ct];
                 const int off = pos % GFA_PAGE;
                 if (head < ex.H + ex.Hkv) {
                     *(uint2*)(ex.k_pages + key_elem(page, head - ex.H, off, d, ex.Hkv, hd)) =
@@ -596,7 +613,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                 e[2] = float_to_bf16(r.z * g.z);
                 e[3] = float_to_bf16(r.w * g.w);
                 *(uint2*)(ex.xg_out + chunked_elem(m, nb + fg * 4, ex.share_rows)) = make_uint2(pk.u.x, pk.u.y);
-                part_ssq += fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
+                part_ssq[ct] += fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
             }
         } else {
 #pragma unroll
@@ -608,9 +625,17 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         }
     }
     if (MODE == 2 && ex.xg_out) {                        // this workgroup's share, rows side by side
-        part_ssq += __shfl_xor(part_ssq, 16, GFA_WAVE);
-        part_ssq += __shfl_xor(part_ssq, 32, GFA_WAVE);
-        if (fg == 0 && fi < ex.share_rows) ex.ssq_out[(size_t)blockIdx.x * ex.share_rows + fi] = part_ssq;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float p = part_ssq[ct];
+            p += __shfl_xor(p, 16, GFA_WAVE);
+            p += __shfl_xor(p, 32, GFA_WAVE);
+            if (fg == 0 && ct * 16 + fi < ex.share_rows)
+                ex.ssq_out[(size_t)blockIdx.x * ex.share_rows + ct * 16 + fi] = p;
+        }
+        // a record is wider than the tiles of rows with 33..48 rows: the rest is zero
+        if (fg == 1 && CT * 16 + fi < ex.share_rows)
+            ex.ssq_out[(size_t)blockIdx.x * ex.share_rows + CT * 16 + fi] = 0.f;
     }
 }
 
@@ -651,12 +676,14 @@ static int pick_tile_rows(int N, int step, int nt = 1) {
     return best_cost * 20 <= cost16 * 19 ? best : 16;
 }
 
-// Tiles of W's rows per workgroup: two for nine to sixteen rows of x where the workgroups
+// Tiles of W's rows per workgroup: two for nine to 48 rows of x where the workgroups
 // still fill three quarters of the chip (measured on 256 compute units at sixteen rows of x:
 // 8192 x 28672 89 -> 79 us, 8192 x 8192 30.6 -> 26.5, 6144 x 4096 14.2 -> 12.8; with 4096 rows
 // of W, 128 workgroups, a loss of a fifth).
 static int tiles_per_workgroup(int mode, int M, int N) {
-    return (mode != 3 && M > 8 && M <= 16 && N >= 24 * compute_units()) ? 2 : 1;
+    // 33..48 rows: only where the registers hold it (the plain epilogues)
+    const int most = (mode == 2 || mode == 4) ? 32 : 48;
+    return (mode != 3 && M > 8 && M <= most && N >= 24 * compute_units()) ? 2 : 1;
 }
 
 // Tile height the launcher below uses for this mode, these rows of x and this width.
@@ -668,7 +695,7 @@ static int tile_rows(int mode, int M, int N) {
 // two-kernel norm's shares are one record per workgroup of mode 2, so its callers size
 // their buffers by it).
 extern "C" int gfa_skinny_workgroups(int mode, int M, int N) {
-    const int per = tile_rows(mode, M, N) * tiles_per_workgroup(mode, M, N);
+    const int per = (M <= 16 ? tile_rows(mode, M, N) : 16) * tiles_per_workgroup(mode, M, N);
     return (N + per - 1) / per;
 }
 
@@ -678,7 +705,7 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     const int ct = (M + 15) / 16;
     // the epilogues that add into the residual stream or rotate pairs work on groups of
     // four columns: their tiles are 12 or 16 rows high
-    const int nt = ct == 1 ? tiles_per_workgroup(MODE, M, N) : 1;
+    const int nt = tiles_per_workgroup(MODE, M, N);
     const int th = ct == 1 ? tile_rows(MODE, M, N) : 16;
     const int tiles = (N + th * nt - 1) / (th * nt);     // workgroups
     const int RT = (MODE == 3) ? 2 : nt;                 // tiles of W staged per wave
@@ -699,8 +726,13 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     }
     SkinnyExtra exl = ex;
     if (ex.ssq_in) {                                     // the waves' pieces for the norm's shares
+        const int per_copy = 64 / ex.share_rows;         // records per copy instruction
+        int copies = (ex.t_in + per_copy * nw - 1) / (per_copy * nw);
+        if (copies > GFA_MAX_SHARE_COPIES) copies = GFA_MAX_SHARE_COPIES;
+        while (copies > 1 && shmem + (size_t)nw * copies * 64 * sizeof(float) > 128 * 1024) --copies;
         exl.share_off = (int)shmem;
-        shmem += (size_t)nw * 16 * 64 * sizeof(float);
+        exl.share_copies = copies;
+        shmem += (size_t)nw * copies * 64 * sizeof(float);
     }
 #define GFA_LAUNCH_MFMA(CTV, XPV, XFV, NTV)                                                            \
     do {                                                                                          \
@@ -719,8 +751,14 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
             else if (nt == 2) GFA_LAUNCH_MFMA(1, 1, true, (MODE == 3 ? 1 : 2));
             else GFA_LAUNCH_MFMA(1, 1, true, 1);
             break;
-        case 2: GFA_LAUNCH_MFMA(2, 1, false, 1); break;
-        case 3: GFA_LAUNCH_MFMA(3, 1, false, 1); break;
+        case 2:
+            if (nt == 2) GFA_LAUNCH_MFMA(2, 1, false, (MODE == 3 ? 1 : 2));
+            else GFA_LAUNCH_MFMA(2, 1, false, 1);
+            break;
+        case 3:
+            if (nt == 2) GFA_LAUNCH_MFMA(3, 1, false, (MODE == 3 ? 1 : 2));
+            else GFA_LAUNCH_MFMA(3, 1, false, 1);
+            break;
         default: GFA_LAUNCH_MFMA(4, 1, false, 1); break;
     }
 #undef GFA_LAUNCH_MFMA
@@ -746,7 +784,7 @@ extern "C" int gfa_skinny_mfma_bf16(const void* x, const void* w, void* out, int
 // Fused q,k,v projection -> rotary encoding -> q_out and the cache pages, one kernel.
 // w [(H + 2 Hkv) hd, K]; head size a multiple of 16, rotary width even, interleaved pairs.
 // x [M <= 64, K] are normed rows; or, with ssq_in [t_in, gfa_share_rows(M)], the two halves of
-// a norm that gfa_skinny_into_chain_bf16 left (eps the norm's; up to 16 rows).
+// a norm that gfa_skinny_into_chain_bf16 left (eps the norm's).
 extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t_in, float eps,
                                        const void* w, void* q_out, void* k_pages, void* v_pages,
                                        const float* freqs, const int* tok_seq, const int* tok_pos,
@@ -769,7 +807,7 @@ extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t
     ex.hd = hd;
     ex.rot = rot;
     if (ssq_in) {                                         // second half of a two-kernel norm
-        if (M > 16 || t_in <= 0) return (int)hipErrorInvalidValue;
+        if (t_in <= 0) return (int)hipErrorInvalidValue;
         ex.ssq_in = ssq_in;
         ex.t_in = t_in;
         ex.share_rows = gfa_share_rows(M);
@@ -780,7 +818,7 @@ extern "C" int gfa_qkv_rope_store_bf16(const void* x, const float* ssq_in, int t
     return launch_skinny_mfma<4>((const bf16_t*)x, (const bf16_t*)w, nullptr, M, N, K, 0, 0, ex, stream);
 }
 
-// residual [M, N] += x w^T for up to 16 rows, and the first half of the norm that follows:
+// residual [M, N] += x w^T for up to 64 rows, and the first half of the norm that follows:
 // xg_out = bfloat16(new residual * next_g), kept chunked ([N / 8][share_rows][8], see
 // chunked_elem), ssq_out [tiles, share_rows] = the workgroups' shares of the rows' sums of
 // squares, tiles = gfa_skinny_workgroups(2, M, N); share_rows = gfa_share_rows(M).
@@ -790,7 +828,7 @@ extern "C" int gfa_skinny_into_chain_bf16(const void* x, int x_chunked, const vo
                                           float* residual, int M, int N, int K, const float* next_g,
                                           void* xg_out, float* ssq_out, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 8 != 0 || N % 8 != 0 || !next_g || !xg_out || !ssq_out)
+    if (M > 64 || K <= 0 || K % 8 != 0 || N % 8 != 0 || !next_g || !xg_out || !ssq_out)
         return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.share_rows = gfa_share_rows(M);
@@ -801,7 +839,7 @@ extern "C" int gfa_skinny_into_chain_bf16(const void* x, int x_chunked, const vo
     return launch_skinny_mfma<2>((const bf16_t*)x, (const bf16_t*)w, residual, M, N, K, N, 0, ex, stream);
 }
 
-// The product that follows: x = xg (M <= 16 rows of K, chunked as the kernel above leaves
+// The product that follows: x = xg (M <= 64 rows of K, chunked as the kernel above leaves
 // them), the result scaled by rsqrt(sum of ssq_in[:, m] / K + eps), ssq_in [t_in,
 // gfa_share_rows(M)].  mode 0 bfloat16 out, 1 float out, 3 gate; out_chunked (gate only, N a
 // multiple of 8): the result is left chunked for the product that reads it next.
@@ -810,7 +848,7 @@ extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, 
                                            int mode, int gate_rows, int out_chunked,
                                            hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 8 != 0 || !ssq_in || t_in <= 0) return (int)hipErrorInvalidValue;
+    if (M > 64 || K <= 0 || K % 8 != 0 || !ssq_in || t_in <= 0) return (int)hipErrorInvalidValue;
     if (out_chunked && (mode != 3 || N % 8 != 0)) return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.ssq_in = ssq_in;

@@ -57,7 +57,7 @@ def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int)
 def attention(q, k_pages, v_pages, batch, table, scale, window, chunked: bool = False):
     """The kernel's result [N, H, hd], or None if it does not take this shape (head sizes
     that are no multiple of 16 or exceed 256 go to the plain kernel).  ``chunked``: where the
-    step is one token for each of up to 16 sequences, the result [N, H * hd] is returned as
+    step is one token for each of up to 64 sequences, the result [N, H * hd] is returned as
     ``gemm_bf16.ChunkedRows``, the order in which the few-row product that follows loads it."""
     n, H, hd = q.shape
     G = k_pages.shape[1]
@@ -83,7 +83,7 @@ def attention(q, k_pages, v_pages, batch, table, scale, window, chunked: bool = 
         return out
     rt, nw, tiles, splits = plan(batch.n_seqs, batch.max_q_len, H, G, hd, table.shape[1])
     one_each = batch.max_q_len == 1 and n == batch.n_seqs
-    chunked = chunked and one_each and n <= 16 and tiles == 1
+    chunked = chunked and one_each and n <= 64 and tiles == 1
     if chunked:
         from .gemm_bf16 import ChunkedRows
         res = ChunkedRows(n, H * hd, q.device)

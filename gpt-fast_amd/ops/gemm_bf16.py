@@ -13,16 +13,16 @@ DOT_MAX_ROWS = 1
 
 
 class ChunkedRows:
-    """Up to 16 rows of bfloat16 as one few-row product leaves them for the next:
-    ``data`` holds [cols / 8][pad][8] (pad = 4, 8 or 16, the least that holds the rows), so
+    """Up to 64 rows of bfloat16 as one few-row product leaves them for the next:
+    ``data`` holds [cols / 8][pad][8] (pad = 4, 8, 16, 32 or 64, the least that holds the rows), so
     that the lanes which load one 16-byte chunk each of different rows read consecutive
     bytes.  Only the kernels of this module look inside; :meth:`to_rows` is for tests."""
 
     __slots__ = ("data", "rows", "cols", "pad")
 
     def __init__(self, rows: int, cols: int, device):
-        if not 0 < rows <= 16 or cols % 8:
-            raise KernelError(f"chunked rows: {rows} x {cols} (1..16 rows, columns in eights)")
+        if not 0 < rows <= MAX_ROWS or cols % 8:
+            raise KernelError(f"chunked rows: {rows} x {cols} (1..{MAX_ROWS} rows, columns in eights)")
         self.rows, self.cols, self.pad = rows, cols, share_rows(rows)
         self.data = torch.empty(cols * self.pad, dtype=torch.bfloat16, device=device)
 
@@ -46,7 +46,7 @@ class ChunkedRows:
 def share_rows(n_rows: int) -> int:
     """Rows per record of the sums-of-squares shares, and per chunk of chunked rows, for this
     many rows of x."""
-    return 4 if n_rows <= 4 else 8 if n_rows <= 8 else 16
+    return 4 if n_rows <= 4 else 8 if n_rows <= 8 else 16 if n_rows <= 16 else 32 if n_rows <= 32 else 64
 
 
 def _entry(M: int, K: int):
@@ -111,16 +111,25 @@ def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor]
     return out
 
 
+# Rows up to which the products of a layer hand their rows to one another (the norms in two
+# halves, the rows chunked); the kernels take up to MAX_ROWS.  Measured on the 8B shape
+# against the vendor library's products with the passes between them: 4.14 -> 3.95 ms per
+# step at 17..24 rows, 4.30 -> 4.22 at 32, 4.60 -> 5.9 at 40 (every workgroup of a consumer
+# reads all shares of the norm, 64 rows wide from 33 rows on).
+CHAIN_MAX_ROWS = 32
+
+
 def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:
-    """The residual-completing product of this shape can prepare the norm that follows."""
-    return 0 < n_rows <= 16 and n_out % 8 == 0 and inner % 8 == 0
+    """The residual-completing product of this shape prepares the norm that follows (where
+    that is the faster way; the kernel itself takes up to MAX_ROWS rows)."""
+    return 0 < n_rows <= CHAIN_MAX_ROWS and n_out % 8 == 0 and inner % 8 == 0
 
 
 def skinny_into_chain(x, w: torch.Tensor, residual: torch.Tensor, next_g: torch.Tensor):
     """residual += x w^T, and the first half of the RMS norm that follows: returns
     ``xg`` = bfloat16(new residual * next_g) as :class:`ChunkedRows` and ``ssq`` float32
     [workgroups, R]: per workgroup (one or two tiles of 12 to 16 columns) its share of each row's sum of
-    squares, R = 4, 8 or 16 rows per record (the least that holds M).  Up to 16 rows; x a
+    squares, R = 4, 8, 16, 32 or 64 rows per record (the least that holds M).  Up to 64 rows; x a
     tensor [M, K] or :class:`ChunkedRows` (the gate's result, left so on request)."""
     chunked = isinstance(x, ChunkedRows)
     _check_operands(x.data.view(x.pad, x.cols)[:x.rows] if chunked else x, w, "skinny_into_chain")
@@ -131,7 +140,7 @@ def skinny_into_chain(x, w: torch.Tensor, residual: torch.Tensor, next_g: torch.
         raise KernelError("skinny_into_chain: residual must be contiguous float32 [M, N]")
     if next_g.dtype != torch.float32 or next_g.numel() != N or not next_g.is_contiguous():
         raise KernelError("skinny_into_chain: one float32 norm weight per column")
-    if not can_chain_norm(M, N, K):
+    if N % 8 or K % 8:                                   # up to MAX_ROWS rows: checked above
         raise KernelError(f"skinny_into_chain: [{M}, {K}] x [{N}, {K}] is outside this kernel")
     xg = ChunkedRows(M, N, w.device)
     records = library("gemm_bf16").gfa_skinny_workgroups(_i(2), _i(M), _i(N))   # one per workgroup

@@ -340,6 +340,8 @@ def test_single_token_attention_in_a_batch(H, G, hd, window):
     entries a wave keeps in registers - on scattered pages with poisoned tails."""
     _single_token_batch(H, G, hd, window, [1, 63, 64, 65, 200, 333, 4100, 2])
     _single_token_batch(H, G, hd, window, [5, 333, 64, 129, 1])        # short: no context split
+    _single_token_batch(H, G, hd, window, [3 + 11 * i for i in range(21)])    # rows chunked by 32
+    _single_token_batch(H, G, hd, window, [70 - i for i in range(40)])        # and by 64
 
 
 def _single_token_batch(H, G, hd, window, lens):
@@ -552,7 +554,7 @@ def test_argmax_and_sampling():
     assert not torch.equal(a, c)
 
 
-@pytest.mark.parametrize("M", [1, 2, 5, 16])
+@pytest.mark.parametrize("M", [1, 2, 5, 16, 17, 31, 33, 48, 64])
 @pytest.mark.parametrize("D,K_,N2,eps", [(72, 40, 48, 1e-5), (200, 328, 208, 1e-6),
                                          (4096, 1024, 256, 1e-5), (1000, 64, 96, 0.3),
                                          (8192, 64, 64, 1e-5)])
@@ -573,7 +575,7 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
     res_ref = res0.double() + y.double() @ wo.double().T
     close(res, res_ref, 1e-5)
     close(ssq.sum(0)[:M], (res.double() ** 2).sum(1), 1e-5)
-    assert ssq.shape[1] == (4 if M <= 4 else 8 if M <= 8 else 16)
+    assert ssq.shape[1] == (4 if M <= 4 else 8 if M <= 8 else 16 if M <= 16 else 32 if M <= 32 else 64)
     assert M == ssq.shape[1] or float(ssq[:, M:].abs().max()) == 0
     n = res.double() * torch.rsqrt((res.double() ** 2).mean(-1, keepdim=True) + eps) * g.double()
     ref = n @ w.double().T
@@ -605,10 +607,10 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
         assert torch.equal(xg_a.to_rows(), xg_b.to_rows())
 
 
-@pytest.mark.parametrize("M", [9, 12, 16])
+@pytest.mark.parametrize("M", [9, 12, 16, 20, 32, 40, 48])
 def test_wide_matrices_at_nine_to_sixteen_rows(M):
     """From 6,144 rows of W on, a workgroup of the few-row kernel takes two tiles of W against
-    the same fragments of x (nine to sixteen rows of x): every epilogue on such a shape, the
+    the same fragments of x (nine to 48 rows of x): every epilogue on such a shape, the
     last workgroup with a second tile that is partly or wholly beyond the matrix."""
     from gpt_fast_amd.ops import gemm_bf16 as G
     torch.manual_seed(M)
@@ -637,9 +639,9 @@ def test_wide_matrices_at_nine_to_sixteen_rows(M):
         close(G.skinny_after_chain(xg, ssq, eps, w2, out_dtype=torch.float32), n @ w2.double().T, 1e-2)
     # projection, rotation and cache write: 64 heads of 128 are 8,192 rows of W
     H, G_, hd = 48, 8, 128
-    pos = [3, 64, 200][:1] * M
     tok_seq = torch.arange(M, dtype=torch.int32, device=DEV)
-    tok_pos = torch.tensor([5 + 7 * i for i in range(M)], dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor([5 + 5 * i for i in range(M)], dtype=torch.int32, device=DEV)
+    assert int(tok_pos.max()) < 4 * 64                     # four pages per sequence
     table = torch.arange(M * 4, dtype=torch.int32, device=DEV).view(M, 4)
     freqs = (1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))).to(DEV)
     xn = bf(torch.randn(M, K_, device=DEV))

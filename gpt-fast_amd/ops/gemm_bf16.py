@@ -112,11 +112,12 @@ def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor]
 
 
 # Rows up to which the products of a layer hand their rows to one another (the norms in two
-# halves, the rows chunked); the kernels take up to MAX_ROWS.  Measured on the 8B shape
-# against the vendor library's products with the passes between them: 4.14 -> 3.95 ms per
-# step at 17..24 rows, 4.30 -> 4.22 at 32, 4.60 -> 5.9 at 40 (every workgroup of a consumer
-# reads all shares of the norm, 64 rows wide from 33 rows on).
-CHAIN_MAX_ROWS = 32
+# halves, the rows chunked); the kernels take up to MAX_ROWS.  Measured against the vendor
+# library's products with the passes between them, per step: 8B shape 4.14 -> 3.95 ms at
+# 17..24 rows, 4.30 -> 4.22 at 32, 4.60 -> 5.9 at 40 (every workgroup of a consumer reads all
+# shares of the norm, 64 rows wide from 33 rows on); 70B shape 26.6 -> 26.5 ms at 24 rows,
+# 27.1 -> 27.8 at 32.
+CHAIN_MAX_ROWS = 24
 
 
 def can_chain_norm(n_rows: int, n_out: int, inner: int) -> bool:

@@ -679,7 +679,9 @@ static int pick_tile_rows(int N, int step, int nt = 1) {
 // Tiles of W's rows per workgroup: two for nine to 48 rows of x where the workgroups
 // still fill three quarters of the chip (measured on 256 compute units at sixteen rows of x:
 // 8192 x 28672 89 -> 79 us, 8192 x 8192 30.6 -> 26.5, 6144 x 4096 14.2 -> 12.8; with 4096 rows
-// of W, 128 workgroups, a loss of a fifth).
+// of W, 128 workgroups, a loss of a fifth).  Not the gate, which multiplies two sets of rows
+// against the same x already: with two tiles of each, 242 registers, the step at sixteen rows
+// lost 5 % (8B and 70B shapes) although the kernel alone gained 3 %.
 static int tiles_per_workgroup(int mode, int M, int N) {
     // 33..48 rows: only where the registers hold it (the plain epilogues)
     const int most = (mode == 2 || mode == 4) ? 32 : 48;

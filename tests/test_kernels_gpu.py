@@ -637,6 +637,12 @@ def test_wide_matrices_at_nine_to_sixteen_rows(M):
         close(xg.to_rows().double() * torch.rsqrt(ssq.sum(0)[:M, None].double() / N + eps), n, 1e-2)
         w2 = bf(torch.randn(8192 + 16, N, device=DEV) * 0.02)
         close(G.skinny_after_chain(xg, ssq, eps, w2, out_dtype=torch.float32), n @ w2.double().T, 1e-2)
+    # the gate: two tiles of W1's rows and their two tiles of W3's rows per workgroup (9..16 rows)
+    for I in (6144, 6152):
+        x = bf(torch.randn(M, K_, device=DEV))
+        w13 = bf(torch.randn(2 * I, K_, device=DEV) * 0.1)
+        a = x.double() @ w13.double().T
+        close(G.skinny_gated(x, w13), (a[:, :I] * torch.sigmoid(a[:, :I])) * a[:, I:], 2e-2)
     # projection, rotation and cache write: 64 heads of 128 are 8,192 rows of W
     H, G_, hd = 48, 8, 128
     tok_seq = torch.arange(M, dtype=torch.int32, device=DEV)

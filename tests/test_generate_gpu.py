@@ -270,8 +270,9 @@ def test_parts_alone(tmp_path_factory):
 @pytest.mark.parametrize("n_seqs", [5, 24, 40])
 def test_graph_replays_equal_eager_steps_for_any_batch_size(tmp_path_factory, n_seqs):
     """The captured step is replayed many times with eager work and synchronisations in
-    between; every replay must give the tokens of the uncaptured step.  24 and 40 rows go
-    through the vendor library's products inside the graph."""
+    between; every replay must give the tokens of the uncaptured step.  24 rows go through
+    the few-row kernels with two tiles of rows, 40 through the vendor library's products
+    inside the graph."""
     from gpt_fast_amd import Entry
     from gpt_fast_amd.engine.decode import DecodeSession
     from gpt_fast_amd.sampling import SamplingParams
@@ -429,27 +430,29 @@ def test_trace_run_chunks_and_a_mixed_step(tmp_path_factory, tmp_path):
                 assert torch.equal(got, whole), r
 
 
-def test_generation_in_bfloat16_with_rows_that_retire_mid_session(tmp_path_factory):
-    """24 requests in batches of 20 and 4, bfloat16, a stop token that ends several requests
-    at different steps: the recorded step is replayed with filler rows in place of the ended
-    requests, over more than sixteen rows (the vendor library's products inside the
-    recording).  The tokens equal those of the same run without a recording."""
+@pytest.mark.parametrize("batch,total", [(20, 24), (28, 32)])
+def test_generation_in_bfloat16_with_rows_that_retire_mid_session(tmp_path_factory, batch, total):
+    """Requests in a batch of 20 (28) and one of 4, bfloat16, a stop token that ends several
+    requests at different steps: the recorded step is replayed with filler rows in place of
+    the ended requests, over more than sixteen rows (20: the few-row kernels with two tiles of
+    rows; 28: the vendor library's products inside the recording).  The tokens equal those of
+    the same run without a recording."""
     import gpt_fast_amd as gfa
     folder = util.make_folder(tmp_path_factory.getbasetemp(), "B")
     cfg = plain.read_config(folder)
-    prompts = [util.random_tokens(cfg["vocab"], 1 + (5 * i) % 31, 500 + i) for i in range(24)]
-    eng = engine_for(folder, "bfloat16", max_tokens=64 * 20)
-    free = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=20,
+    prompts = [util.random_tokens(cfg["vocab"], 1 + (5 * i) % 31, 500 + i) for i in range(total)]
+    eng = engine_for(folder, "bfloat16", max_tokens=64 * batch)
+    free = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=batch,
                         use_graph=False).tokens
     # a token that some requests draw early and others late or never
     counts = {}
     for t in free:
         for tok in set(t[2:20]):
             counts[tok] = counts.get(tok, 0) + 1
-    stop = max(counts, key=lambda k: (min(counts[k], 24 - counts[k]), k))
+    stop = max(counts, key=lambda k: (min(counts[k], total - counts[k]), k))
     runs = {}
     for use_graph in (False, True):
-        res = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=20,
+        res = gfa.generate(eng, prompts, max_new_tokens=24, temperature=0.0, batch_size=batch,
                            stop_tokens=[stop], use_graph=use_graph)
         runs[use_graph] = res
         assert eng.cache.slots.held == 0
@@ -457,12 +460,12 @@ def test_generation_in_bfloat16_with_rows_that_retire_mid_session(tmp_path_facto
     assert runs[True].tokens == runs[False].tokens
     assert runs[True].finish_reasons == runs[False].finish_reasons
     ended = [i for i, r in enumerate(runs[True].finish_reasons) if r == "stop"]
-    assert 2 <= len(ended) < 24
+    assert 2 <= len(ended) < total
     assert len({len(runs[True].tokens[i]) for i in ended}) > 1      # at different steps
     for i in ended:
         assert runs[True].tokens[i][-1] == stop and stop not in runs[True].tokens[i][:-1]
     # sampled, with a seed: also the same with and without the recording
-    kw = dict(max_new_tokens=12, temperature=0.9, top_k=30, batch_size=20, stop_tokens=[stop])
+    kw = dict(max_new_tokens=12, temperature=0.9, top_k=30, batch_size=batch, stop_tokens=[stop])
     a = gfa.generate(eng, prompts, seed=5, use_graph=True, **kw).tokens
     b = gfa.generate(eng, prompts, seed=5, use_graph=False, **kw).tokens
     c = gfa.generate(eng, prompts, seed=6, use_graph=True, **kw).tokens

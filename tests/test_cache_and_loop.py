@@ -394,3 +394,32 @@ def test_attention_plan_for_single_token_steps():
     # 32 query heads on one kv head: two row tiles per token; wide heads: two waves
     assert plan(2, 1, 32, 1, 64, 8)[2] == 2
     assert plan(2, 1, 4, 2, 256, 8)[1] == 2
+
+
+def test_cache_page_order_is_a_permutation():
+    """The order in which a page's keys and values lie (the kernel tests build and read pages
+    through util.key_places / value_places): every element has one place, for head sizes that
+    take the operand order and for those that fall back to rows; and in the operand order the
+    sixteen keys of a score tile and a 16-byte chunk of dims are 256 consecutive bytes."""
+    import torch
+    import util
+    for hd in (16, 20, 24, 48, 64, 128, 256):
+        kp, vp = util.key_places(hd), util.value_places(hd)
+        assert sorted(kp.reshape(-1).tolist()) == list(range(64 * hd))
+        assert sorted(vp.reshape(-1).tolist()) == list(range(64 * hd))
+        k = torch.arange(2 * 3 * 64 * hd, dtype=torch.float32).view(2, 3, 64, hd)
+        v = -torch.arange(2 * 3 * 64 * hd, dtype=torch.float32).view(2, 3, hd, 64)
+        a, b = util.to_cache_order(k, v)
+        k2, v2 = util.from_cache_order(a, b)
+        assert torch.equal(k, k2) and torch.equal(v, v2)
+    kp = util.key_places(128)
+    # tile t of a 32-key block: keys 8 a + 4 t + b; their chunk c lies at slots 16 t .. 16 t + 15
+    for t in (0, 1):
+        keys = [8 * a + 4 * t + b for a in range(4) for b in range(4)]
+        for c in (0, 5, 15):
+            places = [int(kp[32 + k, 8 * c]) for k in keys]
+            assert places == list(range(places[0], places[0] + 128, 8))
+    vp = util.value_places(128)
+    # a value tile: dims 16 j .. 16 j + 15, eight consecutive keys each: 16 bytes per dim, dims side by side
+    assert [int(vp[16 + i, 40]) for i in range(16)] == list(range(int(vp[16, 40]), int(vp[16, 40]) + 128, 8))
+    assert [int(vp[16, 40 + e]) for e in range(8)] == list(range(int(vp[16, 40]), int(vp[16, 40]) + 8))

@@ -270,7 +270,11 @@ extern "C" int gfa_share_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : M <= 16 
 // tiles of W's rows, one below the other, against the same fragments of x.  With sixteen
 // rows every workgroup reads as many bytes of x as of W; two tiles halve that, at half as
 // many workgroups, which pays where those still fill the chip.
-template <int CT, int MODE, int XP = 1, bool XF = false, int TILES = 1>
+// XPL = 2 or 4 (several tiles of x rows, CT > 1): the last tile holds at most eight or four
+// rows, and its idle operand columns carry later steps of k as with XP: with 17 to 24 rows
+// the second tile then takes two load instructions per piece instead of four (a load
+// instruction costs the same whether all its lanes are rows or one is).
+template <int CT, int MODE, int XP = 1, bool XF = false, int TILES = 1, int XPL = 1>
 __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, int th, SkinnyExtra ex) {
@@ -339,6 +343,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
     constexpr int XL = XS / XP;                          // loads of x per piece and tile of rows
     constexpr int XROWS = 16 / XP;
     static_assert(XP == 1 || CT == 1, "shared operand columns need a single tile of rows");
+    static_assert(XPL == 1 || (CT > 1 && XP == 1 && !XF), "a narrower last tile needs several tiles");
+    constexpr int XLL = XS / XPL, XROWSL = 16 / XPL;     // of the last tile of rows
     uint4 x_a[XL][CT], x_b[XL][CT];
     auto load_x = [&](int t, uint4 (&xraw)[XL][CT]) {
 #pragma unroll
@@ -348,6 +354,15 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
                               : t * SM_SUBK + ((XP * s + fi / XROWS) * 4 + fg) * 8;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
+                if (XPL > 1 && ct == CT - 1) {           // the narrower last tile: fewer loads
+                    if (s < XLL) {
+                        const int kl = t * SM_SUBK + ((XPL * s + fi / XROWSL) * 4 + fg) * 8;
+                        const int m = ct * 16 + fi % XROWSL;
+                        const bf16_t* src = ex.x_pad ? x + chunked_elem(m, kl, ex.x_pad) : x + (size_t)m * K + kl;
+                        xraw[s][ct] = (m < M && kl < K) ? *(const uint4*)src : make_uint4(0, 0, 0, 0);
+                    }
+                    continue;
+                }
                 const int m = XF ? ct * 16 + 8 * (s & 1) + (fi & 7) : ct * 16 + fi % XROWS;
                 const bf16_t* src = ex.x_pad ? x + chunked_elem(m, kk, ex.x_pad) : x + (size_t)m * K + kk;
                 xraw[s][ct] = (m < M && kk < K) ? *(const uint4*)src : make_uint4(0, 0, 0, 0);
@@ -381,6 +396,21 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             } else {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) b[ct].u = xraw[s / XP][ct];
+            }
+            if (XPL > 1) {                               // the last tile: its load of this group of steps,
+                uint4 v = xraw[s / XPL][CT - 1];         // rotated down to the step's lanes
+                const int q = s % XPL;
+                if (q * XROWSL == 4) {
+                    v.x = GFA_ROTATE_DOWN(v.x, 4); v.y = GFA_ROTATE_DOWN(v.y, 4);
+                    v.z = GFA_ROTATE_DOWN(v.z, 4); v.w = GFA_ROTATE_DOWN(v.w, 4);
+                } else if (q * XROWSL == 8) {
+                    v.x = GFA_ROTATE_DOWN(v.x, 8); v.y = GFA_ROTATE_DOWN(v.y, 8);
+                    v.z = GFA_ROTATE_DOWN(v.z, 8); v.w = GFA_ROTATE_DOWN(v.w, 8);
+                } else if (q * XROWSL == 12) {
+                    v.x = GFA_ROTATE_DOWN(v.x, 12); v.y = GFA_ROTATE_DOWN(v.y, 12);
+                    v.z = GFA_ROTATE_DOWN(v.z, 12); v.w = GFA_ROTATE_DOWN(v.w, 12);
+                }
+                b[CT - 1].u = v;
             }
             if (XP > 1 && s % XP != 0) {
                 const int q = s % XP;
@@ -736,16 +766,17 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         exl.share_copies = copies;
         shmem += (size_t)nw * copies * 64 * sizeof(float);
     }
-#define GFA_LAUNCH_MFMA(CTV, XPV, XFV, NTV)                                                            \
+#define GFA_LAUNCH_MFMA_L(CTV, XPV, XFV, NTV, XPLV)                                                    \
     do {                                                                                          \
         static bool raised = false;                                                               \
         if (!raised) {                                                                            \
-            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV>,             \
+            hipFuncSetAttribute((const void*)skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV, XPLV>,       \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);          \
             raised = true;                                                                        \
         }                                                                                         \
-        skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, th, exl); \
+        skinny_mfma_kernel<CTV, MODE, XPV, XFV, NTV, XPLV><<<tiles, nw * 64, shmem, stream>>>(x, w, out, M, N, K, ldo, gate_rows, th, exl); \
     } while (0)
+#define GFA_LAUNCH_MFMA(CTV, XPV, XFV, NTV) GFA_LAUNCH_MFMA_L(CTV, XPV, XFV, NTV, 1)
     switch (ct) {
         case 1:                                          // columns of the x operand that stand
             if (M <= 4) GFA_LAUNCH_MFMA(1, 4, false, 1);   // for no row carry later steps of k
@@ -753,9 +784,17 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
             else if (nt == 2) GFA_LAUNCH_MFMA(1, 1, true, (MODE == 3 ? 1 : 2));
             else GFA_LAUNCH_MFMA(1, 1, true, 1);
             break;
-        case 2:
-            if (nt == 2) GFA_LAUNCH_MFMA(2, 1, false, (MODE == 3 ? 1 : 2));
-            else GFA_LAUNCH_MFMA(2, 1, false, 1);
+        case 2:                                          // 17..20, ..24 rows: a narrower second tile
+            if (M <= 20) {
+                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (MODE == 3 ? 1 : 2), 4);
+                else GFA_LAUNCH_MFMA_L(2, 1, false, 1, 4);
+            } else if (M <= 24) {
+                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (MODE == 3 ? 1 : 2), 2);
+                else GFA_LAUNCH_MFMA_L(2, 1, false, 1, 2);
+            } else {
+                if (nt == 2) GFA_LAUNCH_MFMA(2, 1, false, (MODE == 3 ? 1 : 2));
+                else GFA_LAUNCH_MFMA(2, 1, false, 1);
+            }
             break;
         case 3:
             if (nt == 2) GFA_LAUNCH_MFMA(3, 1, false, (MODE == 3 ? 1 : 2));
@@ -764,6 +803,7 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         default: GFA_LAUNCH_MFMA(4, 1, false, 1); break;
     }
 #undef GFA_LAUNCH_MFMA
+#undef GFA_LAUNCH_MFMA_L
     return GFA_LAUNCH_RESULT();
 }
 

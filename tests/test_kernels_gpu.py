@@ -89,7 +89,7 @@ def test_gemm_f32(M, N, K_):
     close(res, keep.double() + ref, 1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 16, 17, 20, 22, 24, 33, 64])
 @pytest.mark.parametrize("N,K_", [(40, 64), (136, 200), (1000, 328), (96, 4096), (77, 75)])
 def test_skinny_bf16(M, N, K_):
     from gpt_fast_amd.ops import gemm_bf16 as G
@@ -554,7 +554,7 @@ def test_argmax_and_sampling():
     assert not torch.equal(a, c)
 
 
-@pytest.mark.parametrize("M", [1, 2, 5, 16, 17, 31, 33, 48, 64])
+@pytest.mark.parametrize("M", [1, 2, 5, 16, 17, 20, 21, 24, 25, 31, 33, 48, 64])
 @pytest.mark.parametrize("D,K_,N2,eps", [(72, 40, 48, 1e-5), (200, 328, 208, 1e-6),
                                          (4096, 1024, 256, 1e-5), (1000, 64, 96, 0.3),
                                          (8192, 64, 64, 1e-5)])
@@ -607,7 +607,7 @@ def test_norm_over_two_kernels(M, D, K_, N2, eps):
         assert torch.equal(xg_a.to_rows(), xg_b.to_rows())
 
 
-@pytest.mark.parametrize("M", [9, 12, 16, 20, 32, 40, 48])
+@pytest.mark.parametrize("M", [9, 12, 16, 18, 20, 23, 24, 32, 40, 48])
 def test_wide_matrices_at_nine_to_sixteen_rows(M):
     """From 6,144 rows of W on, a workgroup of the few-row kernel takes two tiles of W against
     the same fragments of x (nine to 48 rows of x): every epilogue on such a shape, the

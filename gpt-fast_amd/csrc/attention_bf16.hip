@@ -231,9 +231,14 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
             }
 #pragma unroll
             // every tile of dims is multiplied, also those beyond the head (their results are
-            // never stored): with a branch on the head size between the matrix
-            // instructions, the two-tile kernel with prefetch gave wrong sums for its first
-            // tile at head size 16 once a second block of keys was read
+            // never stored).  A test of the head size here (`if (dt * 16 < hd)`) ends a basic
+            // block directly behind a matrix instruction, and for the block it jumps to the
+            // compiler once left out the wait states that the instruction's result needs: on
+            // the path head size 16 takes, the accumulator was copied back
+            // (v_accvgpr_read_b32) three wait states after the instruction instead of seven,
+            // and one of a lane's four sums of the first row tile lost the block's product.
+            // Straight-line code gets its waits; tests/test_isa_hazards.py reads the compiled
+            // kernels for such sequences.
             for (int dt = 0; dt < DT; ++dt)
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
         }
@@ -574,8 +579,8 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
         __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         // every tile of dims is multiplied, also those beyond a smaller head (what LDS holds
-        // there goes into accumulators that are never stored): a branch between matrix
-        // instructions on the same accumulators has given wrong sums
+        // there goes into accumulators that are never stored): no branch directly behind a
+        // matrix instruction (see the wave-level kernel above)
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
             for (int hb = 0; hb < 2; ++hb) {

@@ -332,6 +332,85 @@ def test_attention_finds_one_far_key():
             close(out[0, h], vs[0][target, h // (H // G)].float(), 2e-2)
 
 
+def _chunk_reference(q, k, v, spos, scale):
+    """float64 attention of a chunk q [n, H, hd] at positions spos .. over k, v [S, G, hd]."""
+    n, H, hd = q.shape
+    S, G, _ = k.shape
+    kk = k.double().repeat_interleave(H // G, dim=1)                 # [S, H, hd]
+    vv = v.double().repeat_interleave(H // G, dim=1)
+    s = torch.einsum("nhd,shd->hns", q.double(), kk) * scale
+    mask = torch.arange(S)[None, :] > (spos + torch.arange(n))[:, None]
+    s = s.masked_fill(mask[None], float("-inf"))
+    return torch.einsum("hns,shd->nhd", torch.softmax(s, -1), vv)
+
+
+@pytest.mark.parametrize("hd", [16, 32, 48, 64, 80, 96, 112, 128, 256])
+def test_attention_variants_sweep(hd):
+    """Every instantiation of the matrix-core attention, forced through the C entry points
+    instead of chosen by shape: the wave-level kernel with one, two (the prefetching loop) and
+    four row tiles per wave, one to four waves per workgroup and with the context split over
+    workgroups; the workgroup-tiled kernel in both tile heights; chunks at an offset over one
+    to five pages of keys; one and three query heads per kv head.  In every case some rows
+    have a late key that stands out (a multiple of their own query), so that the running
+    maximum moves - and the output accumulators are rescaled - in a block after the first;
+    the comparison is with float64."""
+    import ctypes
+    from gpt_fast_amd.ops.library import library, ptr, stream_handle
+    lib = library("attention_bf16")
+    i32, f32 = ctypes.c_int, ctypes.c_float
+    scale = 1.0 / math.sqrt(hd)
+    for G, R in ((2, 1), (1, 3)):
+        H = G * R
+        for spos, qlen in [(0, 20), (13, 40), (70, 33), (100, 60), (250, 70)]:
+            S = spos + qlen
+            k_pages, v_pages, table, ks, vs = _paged([S], G, hd, torch.bfloat16, seed=hd + spos)
+            gen = torch.Generator().manual_seed(spos + R)
+            q = bf(torch.randn(qlen, H, hd, generator=gen))
+            # every fourth token's first head of each group: its own position's key is three
+            # times its query, the newest key it sees, in the last block it reads
+            k_rows, v_cols = from_cache_order(k_pages.cpu(), v_pages.cpu())
+            for n in range(1, qlen, 4):
+                pos = spos + n
+                page, off = int(table[0, pos // 64]), pos % 64
+                for g in range(G):
+                    ks[0][pos, g] = q[n, g * R] * 3.0
+                    k_rows[page, g, off] = ks[0][pos, g]
+            k_pages, _ = to_cache_order(k_rows, v_cols)
+            k_pages = k_pages.to(DEV)
+            want = _chunk_reference(q.float(), ks[0].float(), vs[0].float(), spos, scale)
+            q_dev = q.to(DEV)
+            q_start = torch.tensor([0, qlen], dtype=torch.int32, device=DEV)
+            start = torch.tensor([spos], dtype=torch.int32, device=DEV)
+            rows = qlen * R
+            # waves that share a workgroup add their partial results in LDS: at most 64 KB
+            per_wave = 128 + (2 if hd <= 64 else 4 if hd <= 128 else 8) * 2 * 1024
+            cases = [("wave", rt, nw, sp) for rt in (1, 2, 4) for nw, sp in ((1, 1), (2, 1), (4, 3))
+                     if not (rt == 4 and hd > 128) and (nw - 1) * rt * per_wave <= 65536]
+            if hd <= 128:
+                cases += [("tiled", rt, 4, 1) for rt in (1, 2)]
+            for kind, rt, nw, splits in cases:
+                out = torch.full((qlen, H, hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+                if kind == "tiled":
+                    code = lib.gfa_attention_tiled_bf16(
+                        ptr(q_dev), ptr(k_pages), ptr(v_pages), ptr(q_start), ptr(start), ptr(table),
+                        i32(table.shape[1]), ptr(out), i32(qlen), i32(1), i32(H), i32(G), i32(hd),
+                        f32(scale), i32(0), i32(rows), i32(rt), stream_handle())
+                else:
+                    ws_o = torch.empty((splits, qlen * H, hd), dtype=torch.float32, device=DEV)
+                    ws_ml = torch.empty((splits, qlen * H, 2), dtype=torch.float32, device=DEV)
+                    tiles = (rows + 16 * rt - 1) // (16 * rt)
+                    code = lib.gfa_attention_bf16(
+                        ptr(q_dev), ptr(k_pages), ptr(v_pages), ptr(q_start), ptr(start), ptr(table),
+                        i32(table.shape[1]), ptr(out), ptr(ws_o), ptr(ws_ml), i32(qlen), i32(1),
+                        i32(H), i32(G), i32(hd), f32(scale), i32(0), i32(rt), i32(nw), i32(tiles),
+                        i32(splits), i32(0), i32(0), stream_handle())
+                assert code == 0, (kind, rt, nw, splits, code)
+                got = out.cpu().double()
+                assert not torch.isnan(got).any(), (kind, rt, nw, splits, R, spos, qlen)
+                err = float((got - want).abs().max() / want.abs().max())
+                assert err < 1.5e-2, (kind, rt, nw, splits, R, spos, qlen, err)
+
+
 @pytest.mark.parametrize("H,G,hd,window", [(8, 2, 128, 0), (4, 4, 16, 0), (16, 1, 64, 0), (6, 2, 48, 37),
                                            (3, 1, 256, 0), (10, 2, 112, 100), (32, 8, 128, 4000)])
 def test_single_token_attention_in_a_batch(H, G, hd, window):

@@ -105,4 +105,4 @@ def write_safetensors(path: str, tensors: Dict[str, torch.Tensor]) -> None:
         f.write(raw)
         for t in blobs:
             if t.numel():
-                f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes())
+                f.write(t.reshape(-1).view(torch.uint8).numpy().data)      # the bytes as they lie, no copy

@@ -56,32 +56,34 @@ def config_from_dict(c):
 
 
 def read_safetensors(path):
-    """Own reader: 8-byte little-endian header length, JSON header, raw data."""
+    """Own reader: 8-byte little-endian header length, JSON header, raw data.  Values come
+    back as float32 (integers as stored); the file is mapped, not read whole."""
     import numpy as np
-    with open(path, "rb") as f:
-        raw = f.read()
-    n = int.from_bytes(raw[:8], "little")
-    header = json.loads(raw[8:8 + n].decode("utf-8"))
+    mm = np.memmap(path, dtype=np.uint8, mode="r")
+    n = int.from_bytes(mm[:8].tobytes(), "little")
+    header = json.loads(mm[8:8 + n].tobytes().decode("utf-8"))
     base = 8 + n
     out = {}
     for name, meta in header.items():
         if name == "__metadata__":
             continue
         lo, hi = meta["data_offsets"]
-        buf = raw[base + lo:base + hi]
+        buf = mm[base + lo:base + hi]
         dt = meta["dtype"]
         shape = meta["shape"]
         if dt == "F32":
-            t = torch.from_numpy(np.frombuffer(buf, dtype="<f4").copy())
-        elif dt == "BF16":
-            u = np.frombuffer(buf, dtype="<u2").astype(np.uint32) << 16
-            t = torch.from_numpy(u.view(np.float32).copy())
+            t = torch.from_numpy(np.array(buf.view("<f4")))
+        elif dt == "BF16":                      # a bfloat16 is the upper half of a float32
+            u = np.empty(buf.size // 2, dtype=np.uint32)
+            u[:] = buf.view("<u2")
+            u <<= 16
+            t = torch.from_numpy(u.view(np.float32))
         elif dt == "F16":
-            t = torch.from_numpy(np.frombuffer(buf, dtype="<f2").copy()).float()
+            t = torch.from_numpy(np.array(buf.view("<f2"))).float()
         elif dt == "F64":
-            t = torch.from_numpy(np.frombuffer(buf, dtype="<f8").copy())
+            t = torch.from_numpy(np.array(buf.view("<f8")))
         elif dt in ("I32", "I64"):
-            t = torch.from_numpy(np.frombuffer(buf, dtype="<i4" if dt == "I32" else "<i8").copy())
+            t = torch.from_numpy(np.array(buf.view("<i4" if dt == "I32" else "<i8")))
         else:
             raise ValueError(f"{name}: dtype {dt}")
         out[name] = t.reshape(shape)

@@ -28,7 +28,7 @@ from ..config.registry import architecture_of, find_preset, read_model_folder
 from ..sampling import SamplingParams
 from .generate import generate
 from .step import Engine
-from .tokenizer import encode_tokens, get_tokenizer
+from .tokenizer import TokenizerError, encode_tokens, get_tokenizer
 
 
 B_INST, E_INST = "[INST]", "[/INST]"          # generate.py:270
@@ -116,8 +116,11 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
         encoded = None                       # synthetic, needs the vocabulary size
     else:
         eos = getattr(config, "eos_token_id", None) or ()
-        tokenizer = get_tokenizer(str(checkpoint_path), bos=getattr(config, "bos_token_id", None),
-                                  eos=eos[0] if eos else None) if checkpoint_path else None
+        try:
+            tokenizer = get_tokenizer(str(checkpoint_path), bos=getattr(config, "bos_token_id", None),
+                                      eos=eos[0] if eos else None) if checkpoint_path else None
+        except TokenizerError as e:
+            raise SystemExit(str(e))
         if tokenizer is None:
             raise SystemExit("a text prompt needs a tokenizer.model or tokenizer.json in the "
                              "model folder (and sentencepiece or tokenizers); use an integer "

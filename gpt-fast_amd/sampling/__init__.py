@@ -5,7 +5,10 @@ reference's law (generate.py:40-57).
 then ``argmax(p / q)`` with ``q ~ Exp(1)`` - a draw from ``p`` that needs no prefix sums
 and no host synchronisation.  ``temperature == 0`` is an exact argmax (lowest index on
 ties).  The noise is a counter-based function of (seed, request key, position), so a
-request's tokens do not depend on what else is in the batch.
+request's tokens do not depend on what else is in the batch: ``q_i = -log((n_i + 1/2) /
+2^23)`` with ``n_i`` the upper 23 bits of word ``i % 4`` of Philox4x32-10 at counter
+``(i // 4, position of the token being drawn, request key, 0)`` under the key ``(seed's low
+word, seed's high word)`` - anyone can recompute a draw from the logits.
 """
 from dataclasses import dataclass
 from typing import Optional

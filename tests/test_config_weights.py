@@ -302,6 +302,77 @@ def test_text_prompts_start_with_bos(tmp_path):
     assert encode_tokens(get_tokenizer(str(tmp_path)), "w2 w1") == [2, 1]    # no id known: none added
 
 
+def test_sentencepiece_model_in_a_folder(tmp_path):
+    """tokenizer.py:24-39: a ``tokenizer.model`` read with sentencepiece; the model is trained
+    here from a few sentences.  Encoding a text for generation puts its BOS id in front
+    (generate.py:213-217) and decoding gives the text back."""
+    spm = pytest.importorskip("sentencepiece")
+    from gpt_fast_amd.engine.tokenizer import SentencePieceTokenizer, encode_tokens, get_tokenizer
+    corpus = tmp_path / "corpus.txt"
+    words = "the quick brown fox jumps over a lazy dog while seven wizards brew quiet potions".split()
+    lines = [" ".join(words[(i * 3 + j) % len(words)] for j in range(7)) for i in range(200)]
+    corpus.write_text("\n".join(lines) + "\n")
+    spm.SentencePieceTrainer.train(input=str(corpus), model_prefix=str(tmp_path / "tokenizer"),
+                                   vocab_size=60, model_type="bpe", bos_id=1, eos_id=2, unk_id=0,
+                                   minloglevel=2)
+    t = get_tokenizer(str(tmp_path))
+    assert isinstance(t, SentencePieceTokenizer)
+    assert (t.bos_id(), t.eos_id()) == (1, 2)
+    ids = encode_tokens(t, "the lazy fox")
+    assert ids[0] == 1 and 1 not in ids[1:] and all(0 <= i < 60 for i in ids)
+    assert t.decode(ids) == "the lazy fox"
+    assert encode_tokens(t, "the lazy fox", bos=False) == ids[1:]
+
+
+def _write_rank_file(path, merges):
+    import base64
+    ranks = [bytes([b]) for b in range(256)] + [m.encode() for m in merges]
+    path.write_bytes(b"".join(base64.b64encode(b) + b" " + str(r).encode() + b"\n"
+                              for r, b in enumerate(ranks)))
+    return len(ranks)
+
+
+def test_rank_file_tokenizer_merges_by_lowest_rank(tmp_path):
+    """tokenizer.py:41-95: the Llama-3 family's ``tokenizer.model`` is a list of byte strings
+    with their ranks.  The reference hands it to the tiktoken package, which is not installed
+    here, so parity with that package is unpinned; what is checked is the algorithm on a file
+    made here: pieces by the reference's pattern, within a piece the pair of lowest rank
+    first, special tokens behind the ranks in the reference's order."""
+    pytest.importorskip("regex")
+    from gpt_fast_amd.engine.tokenizer import RankFileTokenizer, encode_tokens, get_tokenizer
+    n = _write_rank_file(tmp_path / "tokenizer.model", ["he", "ll", "hell", " w", "lo", "hello"])
+    t = get_tokenizer(str(tmp_path))
+    assert isinstance(t, RankFileTokenizer)
+    he, ll, hell, _w, lo, hello = range(256, 262)
+    assert t.encode("hello") == [hello]                   # a whole piece with a rank of its own
+    # "hellow": he (256), then ll (257), then hell (258), then hello (261); w stays a byte
+    assert t.encode("hellow") == [hello, ord("w")]
+    # "hellx": the same merges up to hell; x stays a byte
+    assert t.encode("hellx") == [hell, ord("x")]
+    # "helo": he first, which leaves l, o to form lo
+    assert t.encode("helo") == [he, lo]
+    # "llo": ll has the lower rank, so lo is never formed
+    assert t.encode("llo") == [ll, ord("o")]
+    # the pattern keeps a leading space with its word: " w" + "orld"
+    assert t.encode("hello world") == [hello, _w, ord("o"), ord("r"), ord("l"), ord("d")]
+    assert t.encode("") == []
+    assert (t.bos_id(), t.eos_id()) == (n, n + 1)
+    assert t.special["<|eot_id|>"] == n + 9 and len(t.special) == 256
+    ids = encode_tokens(t, "hello w\u00f6rld 123")
+    assert ids[0] == n and t.decode(ids[1:]) == "hello w\u00f6rld 123"
+
+
+def test_a_tokenizer_file_that_cannot_be_read_says_why(tmp_path):
+    from gpt_fast_amd.engine.tokenizer import TokenizerError, get_tokenizer
+    assert get_tokenizer(str(tmp_path)) is None                 # no file: no tokenizer, no error
+    (tmp_path / "tokenizer.model").write_bytes(b"\x00\x01 this is neither kind of model")
+    with pytest.raises(TokenizerError, match="tokenizer.model"):
+        get_tokenizer(str(tmp_path))
+    (tmp_path / "tokenizer.json").write_text("{ not json")
+    with pytest.raises(TokenizerError, match="tokenizer.model.*tokenizer.json"):
+        get_tokenizer(str(tmp_path))
+
+
 def test_a_library_is_rebuilt_when_its_source_changes(tmp_path, monkeypatch):
     """The stamp beside a built library holds a hash of source, common header and flags; a
     library whose stamp does not fit is not current."""

@@ -83,6 +83,22 @@ def test_sampled_generation_is_seeded_and_batch_independent(tmp_path_factory):
     # the same requests in batches of two draw the same tokens (noise is per request)
     d = gfa.generate(eng, prompts, seed=7, batch_size=2, **kw).tokens
     assert d == a
+    # every token is the one the reference's law draws (generate.py:40-57) from the plain
+    # logits of the request's own sequence with the sampler's stated noise: argmax(p / q),
+    # p = softmax(top-50(logits / 0.8)).  A sampler that read another row's logits, another
+    # position's or request's noise, or forgot the temperature would draw other tokens.
+    _, w = plain.load_folder(folder)
+    for key, (p, new) in enumerate(zip(prompts, a)):
+        logits = plain.forward(w, cfg, p + new[:-1]).double()
+        for j, tok in enumerate(new):
+            pos = len(p) + j                               # the place of the token being drawn
+            probs = plain.logits_to_probs(logits[pos - 1], temperature=0.8, top_k=50)
+            assert int((probs > 0).sum()) == 50 and probs[tok] > 0
+            race = probs / util.sampler_noise(cfg["vocab"], 7, key, pos)
+            best = int(plain.sample_with_noise(probs, util.sampler_noise(cfg["vocab"], 7, key, pos)))
+            # float32 logits and logf differ from these float64 ones in the last bits: on a
+            # near tie of the race the other contender may win
+            assert tok == best or float(race[tok]) > float(race[best]) * (1 - 1e-4), (key, j, tok, best)
 
 
 def test_long_decoding_and_first_tokens(tmp_path_factory):

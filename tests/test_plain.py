@@ -184,6 +184,68 @@ def test_blocks_are_identity_when_output_projections_vanish():     # model.py:16
     assert torch.allclose(plain.forward(w, CFG, toks), ref, rtol=1e-6, atol=1e-6)
 
 
+def test_rope_frequency_ladder_by_hand():                          # model.py:271
+    """f_i = base^(-2i/hd): written out for sizes where the powers are plain decimals.  An
+    exponent i/hd, (2i+1)/hd or 2i/(hd-2) gives other numbers."""
+    assert torch.allclose(plain.rope_frequencies(8, 10000.0),
+                          torch.tensor([1.0, 0.1, 0.01, 0.001]), rtol=1e-6)
+    assert torch.allclose(plain.rope_frequencies(4, 100.0), torch.tensor([1.0, 0.1]), rtol=1e-6)
+    f = plain.rope_frequencies(128, 500000.0).double()
+    assert f.numel() == 64 and f[0] == 1.0
+    assert torch.allclose(f[1:] / f[:-1], torch.full((63,), 500000.0 ** (-2.0 / 128)).double(), rtol=1e-5)
+    assert abs(float(f[-1]) - 500000.0 ** (-126.0 / 128)) < 1e-9
+    # the angle of pair i at position p is p * f_i (model.py:274-276): pair 1 of head size 8
+    cos, sin = plain.rope_table([5], 8, 10000.0)
+    assert abs(float(cos[0, 1]) - math.cos(0.5)) < 1e-6 and abs(float(sin[0, 1]) - math.sin(0.5)) < 1e-6
+
+
+def test_norms_stand_before_mixer_and_feed_forward():             # model.py:161-164
+    """h = x + attention(norm_a(x)), out = h + ffn(norm_f(h)).  With one branch silenced (the
+    other one's output projection zero), what the block adds to its input does not change
+    when the input is scaled, because the branch sees a normed copy (eps -> 0): with the norm
+    behind the branch or behind the sum, it does.  Each branch alone is that part of its own
+    norm's rows, which tells the two norm weights apart, and the whole block is the second
+    branch on the stream after the first sum."""
+    cfg = dict(CFG, eps=1e-12)
+    w = _tiny_weights(cfg, 3)
+    x = torch.randn(5, cfg["dim"], generator=torch.Generator().manual_seed(4))
+    pos = torch.arange(5)
+    for silenced in ("layers.0.feed_forward.w2.weight", "layers.0.attention.wo.weight"):
+        one = dict(w)
+        one[silenced] = torch.zeros_like(w[silenced])
+        added = plain.block(x, one, 0, cfg, pos) - x
+        assert float(added.abs().max()) > 1e-2
+        for c in (0.25, 8.0):
+            assert torch.allclose(plain.block(c * x, one, 0, cfg, pos) - c * x, added,
+                                  rtol=1e-4, atol=1e-5)
+    p = "layers.0."
+    only_attn = dict(w)
+    only_attn[p + "feed_forward.w2.weight"] = torch.zeros_like(w[p + "feed_forward.w2.weight"])
+    a = plain.attention(plain.rms_norm(x, w[p + "attention_norm.weight"], cfg["eps"]),
+                        w[p + "attention.wqkv.weight"], w[p + "attention.wo.weight"], cfg, pos)
+    assert torch.allclose(plain.block(x, only_attn, 0, cfg, pos) - x, a, rtol=1e-5, atol=1e-6)
+    h = x + a
+    f = plain.feed_forward(plain.rms_norm(h, w[p + "ffn_norm.weight"], cfg["eps"]),
+                           w[p + "feed_forward.w1.weight"], w[p + "feed_forward.w3.weight"],
+                           w[p + "feed_forward.w2.weight"])
+    assert torch.allclose(plain.block(x, w, 0, cfg, pos), h + f, rtol=1e-5, atol=1e-6)
+    swapped = dict(w)
+    swapped[p + "attention_norm.weight"], swapped[p + "ffn_norm.weight"] = \
+        w[p + "ffn_norm.weight"], w[p + "attention_norm.weight"]
+    assert not torch.allclose(plain.block(x, swapped, 0, cfg, pos), h + f, rtol=1e-4, atol=1e-5)
+
+
+def test_gate_saturates_where_the_first_matrix_is_negative():     # model.py:227
+    """silu(w1 x) * (w3 x): a row of w1 that maps x far below zero closes the gate whatever
+    w3 gives; a row of w3 far below zero does not."""
+    x = torch.ones(1, 4)
+    w2 = torch.eye(4)
+    closed = plain.feed_forward(x, torch.full((4, 4), -10.0), torch.full((4, 4), 3.0), w2)
+    assert float(closed.abs().max()) < 1e-10
+    open_ = plain.feed_forward(x, torch.full((4, 4), 3.0), torch.full((4, 4), -10.0), w2)
+    assert float(open_.abs().min()) > 100.0
+
+
 def test_forward_is_causal_and_per_position():
     w = _tiny_weights(CFG, 1)
     a = plain.forward(w, CFG, [3, 7, 1, 9, 4])
@@ -216,3 +278,18 @@ def test_sampling_law():                       # generate.py:40-57
     noise = torch.empty(20000, 3).exponential_(1)
     counts = torch.bincount(plain.sample_with_noise(probs.expand(20000, 3), noise), minlength=3)
     assert torch.allclose(counts / 20000.0, probs, atol=0.015)
+
+
+def test_noise_generator_known_answers():
+    """The tests' own Philox4x32-10 (util.philox4x32_10, with which the GPU tests recompute the
+    sampler's noise) against the known answers published with the generator (Random123's
+    kat_vectors: counter and key all zeros, all ones)."""
+    import util
+    got = [int(x[0]) for x in util.philox4x32_10([0], [0], [0], [0], 0, 0)]
+    assert got == [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]
+    ones = 0xFFFFFFFF
+    got = [int(x[0]) for x in util.philox4x32_10([ones], [ones], [ones], [ones], ones, ones)]
+    assert got == [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]
+    q = util.sampler_noise(1001, seed=7, key=3, pos=12)
+    assert q.shape == (1001,) and bool((q > 0).all()) and bool(torch.isfinite(q).all())
+    assert abs(float(q.mean()) - 1.0) < 0.1                      # Exp(1)

@@ -128,3 +128,33 @@ def from_cache_order(k_pages, v_pages):
     k = k_pages.reshape(n, G, -1)[..., key_places(hd).reshape(-1)].view(n, G, 64, hd)
     v = v_pages.reshape(n, G, -1)[..., value_places(hd).reshape(-1)].view(n, G, hd, 64)
     return k, v
+
+
+# The sampler's noise, written again from its description (gpt_fast_amd/sampling): a request's
+# draw at sequence position ``pos`` compares p_i / q_i with q_i = -log(u_i), u_i = (n_i + 1/2) /
+# 2^23, n_i the upper 23 bits of word i % 4 of Philox4x32-10 (Salmon et al., "Parallel random
+# numbers: as easy as 1, 2, 3") with counter (i // 4, pos, request key, 0) and key (seed's low
+# word, seed's high word).
+def philox4x32_10(c0, c1, c2, c3, k0, k1):
+    import numpy as np
+    c0, c1, c2, c3 = (np.asarray(c, dtype=np.uint64) for c in (c0, c1, c2, c3))
+    mask = np.uint64(0xFFFFFFFF)
+    k0, k1 = np.uint64(k0), np.uint64(k1)
+    for _ in range(10):
+        p0 = np.uint64(0xD2511F53) * c0
+        p1 = np.uint64(0xCD9E8D57) * c2
+        c0, c1, c2, c3 = (p1 >> np.uint64(32)) ^ c1 ^ k0, p1 & mask, (p0 >> np.uint64(32)) ^ c3 ^ k1, p0 & mask
+        k0 = (k0 + np.uint64(0x9E3779B9)) & mask
+        k1 = (k1 + np.uint64(0xBB67AE85)) & mask
+    return c0, c1, c2, c3
+
+
+def sampler_noise(vocab, seed, key, pos):
+    """float64 [vocab]: the q_i of one draw."""
+    import numpy as np
+    blocks = np.arange((vocab + 3) // 4, dtype=np.uint64)
+    same = np.zeros_like(blocks)
+    words = philox4x32_10(blocks, same + np.uint64(pos), same + np.uint64(key), same,
+                          seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
+    n = np.stack(words, axis=1).reshape(-1)[:vocab] >> np.uint64(9)
+    return torch.from_numpy(-np.log((n.astype(np.float64) + 0.5) / 8388608.0))

@@ -13,8 +13,10 @@ the live sequences) per second with the HBM peak; ``points`` holds decode at bat
 Other workloads of the same program: ``--preset`` (another shape), ``--context`` (cache
 positions per sequence), ``--prompt-lens LO:HI`` (prompts of unequal, seeded random lengths;
 adds the ragged prefill's tokens per second), ``--prefill-only`` (just the timed prompt, for
-profiling), ``--ceilings`` (what this GPU reaches with a bare read stream and a bare
-matrix-instruction loop, beside the datasheet peaks).
+profiling).  The line also holds what this GPU reaches with a bare read stream and a bare
+matrix-instruction loop (``measured_peaks``, and the step's fractions of them beside the
+fractions of the datasheet peaks), the per-step time of each of the ``--runs`` timed regions
+(``ms_per_step`` is their median) and the peak device memory in use.
 """
 import argparse
 import json
@@ -35,9 +37,11 @@ def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=False):
-    """(seconds per step, bytes a step reads, seconds of the prefill) for ``steps`` decode
-    steps of sequences with the given prompt lengths."""
+def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=False, runs=3):
+    """(seconds per step, bytes a step reads, seconds of the prefill, seconds per step of
+    every run) for decode steps of sequences with the given prompt lengths: ``warmup``
+    untimed steps, then ``runs`` timed regions of exactly ``steps`` steps each, one after
+    the other in the same session; the first figure is the median region's."""
     import torch
     from gpt_fast_amd import Entry
     from gpt_fast_amd.engine.decode import DecodeSession
@@ -73,23 +77,27 @@ def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=
     torch.cuda.synchronize()
     prefill_seconds = time.perf_counter() - t0
     sess = DecodeSession(engine, slots, list(range(batch)), first, params, use_graph=use_graph,
-                         max_new_tokens=warmup + steps + 1)
+                         max_new_tokens=warmup + runs * steps + 1)
     for _ in range(warmup):
         sess.advance()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        sess.advance()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
+    per_run = []
+    for _ in range(runs):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            sess.advance()
+        torch.cuda.synchronize()
+        per_run.append((time.perf_counter() - t0) / steps)
+    median_run = sorted(range(runs), key=lambda r: per_run[r])[runs // 2]
+    dt = per_run[median_run]
     sess.close()
-    # bytes of the middle step: weights once + keys and values of every live token
-    ctx = sum(n + warmup + steps // 2 for n in prompt_lens)
+    # bytes of the median run's middle step: weights once + keys and values of every live token
+    ctx = sum(n + warmup + median_run * steps + steps // 2 for n in prompt_lens)
     kv_bytes = sum(g.bytes_per_token() for _, g in engine.cache.kv_groups) * ctx
     step_bytes = engine.model.parameter_bytes() + kv_bytes
     for s in slots:
         engine.end_sequence(s)
-    return dt, step_bytes, prefill_seconds
+    return dt, step_bytes, prefill_seconds, per_run
 
 
 def prefill_run(engine, n_tokens, repeats=3):
@@ -111,16 +119,6 @@ def prefill_run(engine, n_tokens, repeats=3):
     return sorted(times)[len(times) // 2]          # median
 
 
-def prefill_flops(cfg, n_layers, T):
-    D, H, G, hd, I, V = (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads,
-                         cfg.head_dim, cfg.intermediate_size, cfg.vocab_size)
-    per_layer = (H + 2 * G) * hd * D + H * hd * D + 3 * I * D
-    linear = 2.0 * T * n_layers * per_layer
-    attn = n_layers * 2.0 * 2.0 * H * hd * (T * (T + 1) / 2)      # causal QK^T and PV
-    head = 2.0 * D * V                                             # last row only
-    return linear + attn + head
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,8 +135,8 @@ def main():
     ap.add_argument("--context", type=int, default=4096, help="cache positions per sequence")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the timed prompt")
     ap.add_argument("--prefill-only", action="store_true", help="time the prompt and nothing else")
-    ap.add_argument("--ceilings", action="store_true",
-                    help="also measure a bare read stream, a copy and a matrix-instruction loop")
+    ap.add_argument("--runs", type=int, default=3,
+                    help="timed regions of --steps steps each; the median one is reported")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
     args = ap.parse_args()
@@ -151,10 +149,12 @@ def main():
 
     arch, cfg = gfa.find_preset(args.preset, args.architecture)
     raw = arch.config_dict(cfg)
-    full_layers = raw["num_hidden_layers"]
+    full_layers = raw[arch.layer_count_key]
     if args.layers:
-        raw["num_hidden_layers"] = args.layers
+        raw[arch.layer_count_key] = args.layers
         cfg = arch.read_config(raw)
+    sizes = dict(arch.describe(cfg)) if arch.describe is not None else {}
+    n_layers = raw[arch.layer_count_key]
     batch, context = args.batch, args.context
     if args.prompt_lens:
         lo, hi = (int(v) for v in args.prompt_lens.split(":"))
@@ -175,32 +175,37 @@ def main():
     model_name = "Llama-3.1-8B" if args.preset == "llama-3.1-8b" else args.preset
     # the reference's published number is for this shape only
     headline = args.preset == "llama-3.1-8b" and not args.layers
-    rs = dict(cfg.rope_scaling) if cfg.rope_scaling else None
-    scaling = "none" if not rs else " ".join(
-        [str(rs.get("rope_type", rs.get("type", "")))] + [f"{k} {rs[k]:g}" for k in
-         ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
-         if k in rs])
     use_graph = not args.no_graph
     T = args.prefill_tokens
 
     def prefill_point():
         pt = prefill_run(engine, T)
-        flops = prefill_flops(cfg, cfg.num_hidden_layers, T)
+        flops = engine.model.step_flops([T], [0], n_want=1)      # what the parts count
         log(f"[bench] prefill {T}: {pt * 1e3:.2f} ms")
         return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                 "frac": round(flops / pt / 1e12 / MFMA_PEAK_TFLOPS["bf16"], 4)}
 
+    def with_measured(point, measured):
+        point["frac_of_measured"] = round(point["frac"] * MFMA_PEAK_TFLOPS["bf16"]
+                                          / measured["mfma_bf16_tflops"], 4)
+        return point
+
     if args.prefill_only:
         print(json.dumps({"metric": f"prefill tok/s @ {T} tokens; {model_name} bf16",
-                          "n_layer": cfg.num_hidden_layers, "prefill": prefill_point()}), flush=True)
+                          "n_layer": n_layers, "prefill": prefill_point()}), flush=True)
         return
 
-    if max(prompt_lens) + args.warmup + args.steps + 1 > context:
-        print(f"prompt ({max(prompt_lens)}) + {args.warmup + args.steps + 1} decoded tokens exceed "
-              f"--context {context}")
+    runs = max(1, args.runs)
+    if max(prompt_lens) + args.warmup + runs * args.steps + 1 > context:
+        print(f"prompt ({max(prompt_lens)}) + {args.warmup + runs * args.steps + 1} decoded tokens "
+              f"exceed --context {context}")
         sys.exit(2)
-    dt, step_bytes, prefill_s = decode_run(engine, prompt_lens, args.warmup, args.steps, use_graph,
-                                           warm_prefill=bool(args.prompt_lens))
+    from gpt_fast_amd.ops import ceilings
+    measured = ceilings.measure("cuda:0")          # a few milliseconds of bare kernels
+    log(f"[bench] this GPU: {measured}")
+    dt, step_bytes, prefill_s, per_run = decode_run(engine, prompt_lens, args.warmup, args.steps,
+                                                    use_graph, warm_prefill=bool(args.prompt_lens),
+                                                    runs=runs)
     value = batch / dt
     log(f"[bench] decode b{batch}: {dt * 1e3:.3f} ms/step, {value:.1f} tok/s")
     out = {
@@ -210,21 +215,21 @@ def main():
         "vs_baseline": round(value / BASELINE_TOK_S, 3) if headline and batch == 1 else None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
-            "model": args.preset, "n_layer": cfg.num_hidden_layers,
-            "n_layer_full": full_layers, "dim": cfg.hidden_size,
-            "n_head": cfg.num_attention_heads, "n_kv_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size,
-            "vocab_size": cfg.vocab_size, "rope_base": cfg.rope_theta,
-            "rope_scaling": scaling,
-            "norm_eps": cfg.rms_norm_eps, "global_batch": batch, "seq_len": context,
+            "model": args.preset, **sizes, "n_layer_full": full_layers,
+            "global_batch": batch, "seq_len": context,
             "prompt_len": args.prompt_lens or args.prompt_len,
             "new_tokens": args.warmup + args.steps,
             "weights": "random N(0,0.02) bf16", "sampling": "greedy", "hip_graph": use_graph,
             "parallelism": "single GPU",
         },
+        # ms_per_step is the median of these timed regions of `steps` steps each
+        "runs_ms_per_step": [round(t * 1e3, 4) for t in per_run],
         "roofline": {"bound": "hbm", "achieved": round(step_bytes / dt / 1e9, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)},
+                     "frac": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4),
+                     # what a bare read stream reaches on this GPU, and the step against that
+                     "measured_peak": measured["hbm_read_gbs"],
+                     "frac_of_measured": round(step_bytes / dt / 1e9 / measured["hbm_read_gbs"], 4)},
     }
     if args.prompt_lens:
         # the unequal prompts went through the engine in one step per eight of them (timed on
@@ -233,11 +238,12 @@ def main():
                                  "tokens": sum(prompt_lens), "ms": round(prefill_s * 1e3, 3),
                                  "lengths": " ".join(map(str, prompt_lens))}
     if not args.no_points:
-        out["prefill"] = prefill_point()
+        out["prefill"] = with_measured(prefill_point(), measured)
         points = {}
         for b in (1, 64):
             steps = min(args.steps, 128)
-            d, _, _ = decode_run(engine, [args.prompt_len] * b, min(args.warmup, 8), steps, use_graph)
+            d, _, _, _ = decode_run(engine, [args.prompt_len] * b, min(args.warmup, 8), steps, use_graph,
+                                    runs=runs)
             points[f"decode_b{b}"] = round(b / d, 2)
             log(f"[bench] decode b{b}: {d * 1e3:.3f} ms/step, {b / d:.1f} tok/s")
         out["points"] = points
@@ -245,12 +251,8 @@ def main():
             # like for like: the reference's published number is its batch-1 decode speed
             out["vs_baseline"] = round(points["decode_b1"] / BASELINE_TOK_S, 3)
             out["vs_baseline_point"] = "decode_b1"
-    if args.ceilings:
-        from gpt_fast_amd.ops import ceilings
-        c = ceilings.measure("cuda:0")
-        c["decode_frac_of_read_stream"] = round(step_bytes / dt / 1e9 / c["hbm_read_gbs"], 4)
-        out["ceilings"] = c
-        log(f"[bench] ceilings: {c}")
+    out["measured_peaks"] = measured
+    out["memory_gb"] = round(torch.cuda.max_memory_allocated() / 1e9, 2)
     print(json.dumps(out), flush=True)
 
 

@@ -138,6 +138,20 @@ def llama_native_layouts(c: LlamaConfig):
     return (layout(True), layout(False))
 
 
+def llama_sizes(c: LlamaConfig) -> dict:
+    """Every size and constant of the configuration, flat, under the reference's names
+    (model.py:21-34)."""
+    rs = dict(c.rope_scaling) if c.rope_scaling else None
+    scaling = "none" if not rs else " ".join(
+        [str(rs.get("rope_type", rs.get("type", "")))] + [f"{k} {rs[k]:g}" for k in
+         ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
+         if k in rs])
+    return {"n_layer": c.num_hidden_layers, "dim": c.hidden_size, "n_head": c.num_attention_heads,
+            "n_kv_heads": c.num_key_value_heads, "head_dim": c.head_dim,
+            "intermediate_size": c.intermediate_size, "vocab_size": c.vocab_size,
+            "rope_base": c.rope_theta, "rope_scaling": scaling, "norm_eps": c.rms_norm_eps}
+
+
 LLAMA = register_architecture(Architecture(
     names=("LlamaForCausalLM", "llama"),
     read_config=LlamaConfig.from_dict,
@@ -146,4 +160,5 @@ LLAMA = register_architecture(Architecture(
     config_dict=LlamaConfig.to_dict,
     presets=LlamaConfig.from_name,
     other_layouts=llama_native_layouts,
+    describe=llama_sizes,
 ))

@@ -30,6 +30,11 @@ class Architecture:
     # typed configuration -> further CheckpointLayouts under which the same parameters may
     # be stored (other tensor names); the loader takes the one that fits the files' names
     other_layouts: Callable[[object], tuple] = None
+    # typed configuration -> every size and constant under a short name, flat (numbers and
+    # strings only), for reports and benchmark records
+    describe: Callable[[object], dict] = None
+    # the config.json key that holds the number of layers (a benchmark may run fewer)
+    layer_count_key: str = "num_hidden_layers"
 
     def layouts(self, config) -> tuple:
         """Every layout a checkpoint of ``config`` may have; the first is the one that

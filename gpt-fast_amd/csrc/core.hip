@@ -424,7 +424,7 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     float* qs = shared;                 // [hd]
     float* sc = shared + hd;            // [AG_THREADS]
     float* scratch = sc + AG_THREADS;   // [16]
-    const int h = blockIdx.x, n = blockIdx.y;
+    const int n = blockIdx.x, h = blockIdx.y;     // tokens in x: a step may bring millions
     const int g = h / (H / Hkv);
     const int pos = tok_pos[n];
     const int* pages = table + (size_t)tok_seq[n] * table_stride;
@@ -485,8 +485,8 @@ extern "C" int gfa_attention_generic(const void* q, const void* k_pages, const v
                                      int hd, float scale, int window, int is_bf16,
                                      hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (hd > AG_THREADS * AG_MAX_PER_THREAD) return (int)hipErrorInvalidValue;
-    dim3 grid(H, n_tokens);
+    if (hd > AG_THREADS * AG_MAX_PER_THREAD || H > 65535) return (int)hipErrorInvalidValue;
+    dim3 grid(n_tokens, H);
     const size_t shmem = (size_t)(hd + AG_THREADS + 16) * sizeof(float);
     if (is_bf16)
         attention_generic_kernel<bf16_t><<<grid, AG_THREADS, shmem, stream>>>(
@@ -629,6 +629,7 @@ __global__ void gemm_bf16_naive_kernel(const bf16_t* __restrict__ a, const bf16_
 extern "C" int gfa_gemm_bf16_naive(const void* a, const void* w, float* out, int M, int N, int K,
                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (M > 65535) return (int)hipErrorInvalidValue;     // rows ride in the grid's second dimension
     dim3 grid((N + 255) / 256, M);
     gemm_bf16_naive_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, out, M, N, K);
     return GFA_LAUNCH_RESULT();

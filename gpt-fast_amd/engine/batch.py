@@ -6,7 +6,8 @@ its position, where that sequence's cache pages are) is laid out in one int32 bu
 that goes to the device in a single copy:
 
     tokens[N] tok_seq[N] tok_pos[N] q_start[B+1] start_pos[B] slots[B] row_keys[B]
-    want_rows[W] want_pos[W] seed[2] table_g[B, P_g] for every KV group g
+    want_rows[W] want_pos[W] seed[2] <fields that parts ask for> table_g[B, P_g] for every
+    paged cache group g
 
 ``tok_seq[n]`` is the index of token n's sequence in this batch, ``tok_pos[n]`` its
 position in that sequence (tokens cached before the step + offset in the run);
@@ -14,14 +15,16 @@ position in that sequence (tokens cached before the step + offset in the run);
 sequence b in group g; ``want_rows`` are the indices of the tokens whose logits are wanted and
 ``want_pos`` their positions; ``slots[b]`` is the sequence's slot, which indexes the fixed-size
 state of mixers that keep some; ``seed`` holds the two words of the sampler's seed for
-steps whose sampling is recorded and replayed.
+steps whose sampling is recorded and replayed.  A part that needs something else of the step
+on the device (cumulative lengths, a ring index, ...) declares a :class:`StepField`; the
+model collects them and every step fills and uploads them with the rest.
 
 The reference's step takes ``idx[B, S]`` and one shared ``input_pos[S]`` (model.py:136)
 and a dense ``[Smax, Smax]`` mask (model.py:134); here lengths differ per sequence and
 the mask is implied by ``tok_pos``.
 """
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Callable, Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -42,6 +45,18 @@ class Entry:
     key: int = 0             # identifies the request to the sampler's noise
 
 
+@dataclass(frozen=True)
+class StepField:
+    """A further int32 field of the step's description, asked for by a part (its
+    ``step_fields()``): ``count(n_tokens, n_seqs)`` numbers, written on the host by
+    ``fill(view, entries, starts, cache)`` (``starts[b]`` = tokens cached before the step;
+    an entry whose ``slot`` is None is a filler row).  The part reads it as
+    ``batch.<name>`` (device) or ``batch.host_field(name)``."""
+    name: str
+    count: Callable[[int, int], int]
+    fill: Callable
+
+
 def _round_up(n: int, k: int) -> int:
     return (n + k - 1) // k * k
 
@@ -49,14 +64,23 @@ def _round_up(n: int, k: int) -> int:
 class BatchLayout:
     """Offsets of the fields in the int32 buffer for given counts."""
 
-    def __init__(self, n_tokens: int, n_seqs: int, n_want: int, table_widths: Dict[int, int]):
+    def __init__(self, n_tokens: int, n_seqs: int, n_want: int, table_widths: Dict[int, int],
+                 extra: Sequence[StepField] = ()):
         self.n_tokens, self.n_seqs, self.n_want = n_tokens, n_seqs, n_want
         self.table_widths = dict(table_widths)
+        self.extra = tuple(extra)
         off = 0
         self.fields = {}
-        for name, count in (("tokens", n_tokens), ("tok_seq", n_tokens), ("tok_pos", n_tokens),
-                            ("q_start", n_seqs + 1), ("start_pos", n_seqs), ("slots", n_seqs),
-                            ("row_keys", n_seqs), ("want_rows", n_want), ("want_pos", n_want), ("seed", 2)):
+        own = [("tokens", n_tokens), ("tok_seq", n_tokens), ("tok_pos", n_tokens),
+               ("q_start", n_seqs + 1), ("start_pos", n_seqs), ("slots", n_seqs),
+               ("row_keys", n_seqs), ("want_rows", n_want), ("want_pos", n_want), ("seed", 2)]
+        for f in self.extra:
+            if f.name in dict(own) or f.name in ("buffer", "host", "layout", "table"):
+                raise ValueError(f"a part's step field cannot be named '{f.name}'")
+            own.append((f.name, int(f.count(n_tokens, n_seqs))))
+        for name, count in own:
+            if name in self.fields:
+                raise ValueError(f"two parts ask for a step field named '{name}'")
             self.fields[name] = (off, count)
             off = _round_up(off + count, 4)          # 16-byte aligned fields
         self.tables = {}
@@ -66,7 +90,8 @@ class BatchLayout:
         self.size = max(off, 4)
 
     def key(self):
-        return (self.n_tokens, self.n_seqs, self.n_want, tuple(sorted(self.table_widths.items())))
+        return (self.n_tokens, self.n_seqs, self.n_want, tuple(sorted(self.table_widths.items())),
+                tuple(f.name for f in self.extra))
 
 
 class StepBatch:
@@ -131,17 +156,15 @@ def fill_host(layout: BatchLayout, host: np.ndarray, entries: Sequence[Entry],
             w += 1
         n += q
     host[f["q_start"][0] + len(entries)] = n
+    for field in layout.extra:
+        off, count = f[field.name]
+        field.fill(host[off:off + count], entries, starts, cache)
     if cache is not None:
         for gid, (off, _) in layout.tables.items():
             width = layout.table_widths[gid]
-            for b, e in enumerate(entries):
-                row = host[off + b * width: off + (b + 1) * width]
-                if e.slot is None:                    # a row that only fills the batch's shape
-                    row[:] = cache.groups[gid].spare_page
-                    continue
-                pages = cache.page_list(gid, e.slot)
-                row[:len(pages)] = pages
-                row[len(pages):] = -1
+            group = cache.groups[gid]
+            for b, e in enumerate(entries):           # slot None: a row that only fills the shape
+                group.fill_table_row(host[off + b * width: off + (b + 1) * width], e.slot)
 
 
 class BatchUploader:
@@ -149,8 +172,9 @@ class BatchUploader:
 
     RING = 4
 
-    def __init__(self, device):
+    def __init__(self, device, extra: Sequence[StepField] = ()):
         self.device = torch.device(device)
+        self.extra = tuple(extra)
         self._ring: List[Optional[tuple]] = [None] * self.RING
         self._next = 0
 
@@ -173,10 +197,10 @@ class BatchUploader:
         n_tokens = sum(len(e.tokens) for e in entries)
         n_want = sum(len(e.want) for e in entries)
         widths = {}
-        for gid, _ in cache.kv_groups:
-            most = max(len(cache.page_list(gid, e.slot)) for e in entries)
+        for gid, group in cache.paged_groups:
+            most = max(group.table_entries(e.slot) for e in entries)
             widths[gid] = _round_up(max(most, 1), table_multiple)
-        layout = BatchLayout(n_tokens, len(entries), n_want, widths)
+        layout = BatchLayout(n_tokens, len(entries), n_want, widths, self.extra)
         pinned, event = self._staging(layout.size)
         host = pinned.numpy()[:layout.size]
         fill_host(layout, host, entries, starts, cache)

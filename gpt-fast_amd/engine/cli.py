@@ -24,7 +24,9 @@ from typing import List, Optional, Union
 
 import torch
 
+from ..cache.store import pages_for
 from ..config.registry import architecture_of, find_preset, read_model_folder
+from ..ops.kernels import PAGE
 from ..sampling import SamplingParams
 from .generate import generate
 from .step import Engine
@@ -137,7 +139,10 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
             stream = sys.stdout
         max_seq_length = max_seq_length or INTERACTIVE_POSITIONS
     per_seq = max_seq_length or (prompt_length + max_new_tokens)
-    per_seq = (per_seq + 63) // 64 * 64
+    per_seq = pages_for(per_seq) * PAGE                # the cache is handed out in whole pages
+    most = getattr(arch.plan(config), "max_positions", None)
+    if interactive and most is not None:
+        per_seq = min(per_seq, most)                   # the model's own positions bound a dialogue
     if interactive:
         max_new_tokens = max(1, min(max_new_tokens, per_seq - prompt_length))
     if prompt_length + max_new_tokens > per_seq:
@@ -165,10 +170,6 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
     result = None
     for i in range(-1, num_samples):                       # sample -1 warms up, generate.py:352
         torch.cuda.synchronize()
-        prof = None
-        if profile is not None and i == num_samples - 1:
-            prof = torch.profiler.profile()
-            prof.__enter__()
         new_tokens = max_new_tokens
         callback = None
         if interactive and i >= 0:
@@ -181,7 +182,11 @@ def main(prompt: Union[int, str, List[int]] = "Hello, my name is", num_samples: 
                     f"prompt and answer (--max_seq_length)")
                 continue
             new_tokens = min(max_new_tokens, per_seq - len(encoded))
-            callback = _streamer(tokenizer, stream)
+            callback = _streamer(tokenizer, stream, engine.model.plan.stop_tokens)
+        prof = None
+        if profile is not None and i == num_samples - 1:      # the last sample, generate.py:380-385
+            prof = torch.profiler.profile()
+            prof.__enter__()
         t0 = time.perf_counter()
         result = generate(engine, [encoded] * batch_size, new_tokens,
                           temperature=temperature, top_k=top_k, seed=seed + max(i, 0),
@@ -232,8 +237,12 @@ class _streamer:
     a tokenizer that drops the space in front of a first word keeps it here (the reference
     does this with the id of '.')."""
 
-    def __init__(self, tokenizer, stream, every: int = 4):
+    def __init__(self, tokenizer, stream, stop_tokens=(), every: int = 4):
         self.tokenizer, self.stream, self.every = tokenizer, stream, every
+        # what ends a request: the ids generation stops on, and the tokenizer's own end id
+        self.stop = set(int(t) for t in stop_tokens or ())
+        if tokenizer.eos_id() is not None:
+            self.stop.add(tokenizer.eos_id())
         lead = tokenizer.encode(".")
         self.lead = lead[:1]
         self.cut = len(tokenizer.decode(self.lead)) if self.lead else 0
@@ -245,7 +254,7 @@ class _streamer:
             return
         token = tokens[rows.index(0)]
         self.buffer.append(self.tokenizer.decode(self.lead + [token])[self.cut:])
-        if token == self.tokenizer.eos_id():
+        if token in self.stop:
             self.done = True
         if len(self.buffer) == self.every or self.done:
             self.flush()

@@ -27,6 +27,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from ..sampling import SamplingParams, sample
+from ..cache.store import pages_for
 from .batch import BatchLayout, Entry, StepBatch, fill_host
 
 
@@ -39,7 +40,7 @@ class RecordedStep:
         dev = engine.rt.device
         self.key = step_key(n_rows, widths, params)
         self.params = params
-        self.layout = BatchLayout(n_rows, n_rows, n_rows, widths)
+        self.layout = BatchLayout(n_rows, n_rows, n_rows, widths, engine.step_fields)
         self.staged = [torch.empty(self.layout.size, dtype=torch.int32, pin_memory=True)
                        for _ in range(self.RING)]
         self.staged_events = [None] * self.RING
@@ -50,6 +51,15 @@ class RecordedStep:
         self.tokens = torch.zeros(n_rows, dtype=torch.int32, device=dev)      # fed next
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.busy = False
+
+
+def table_width(pages: int, most: int) -> int:
+    """Entries per row of a session's page table for sequences that grow to ``pages`` pages:
+    the next power of two (at most ``most``, the pool's pages, and never below ``pages``), so
+    that sessions of similar lengths share one recording instead of recording one for every
+    64 tokens of difference."""
+    width = 1 << max(pages - 1, 0).bit_length()
+    return max(pages, min(width, most))
 
 
 def step_key(n_rows: int, widths, params: SamplingParams):
@@ -117,12 +127,12 @@ class DecodeSession:
         if lo < 0 or hi >= engine.vocab_size:
             raise ValueError(f"token ids must lie in [0, {engine.vocab_size}), got {lo}..{hi}")
         widths = {}
-        for gid, _ in self.cache.kv_groups:
+        for gid, group in self.cache.paged_groups:
             most = 1
             for s in self.slots:
                 final = self.cache.length(s) + (max_new_tokens or 0) + 1
-                most = max(most, (final + 63) // 64, len(self.cache.page_list(gid, s)) + 1)
-            widths[gid] = most
+                most = max(most, pages_for(final), group.table_entries(s) + 1)
+            widths[gid] = table_width(most, self.cache.n_pages)
         self.rec = engine.recorded_steps.take(B, widths, params)
         self.layout = self.rec.layout
         self.tokens = self.rec.tokens
@@ -161,9 +171,9 @@ class DecodeSession:
         starts_live = iter(self.cache.extend_many(live)) if live else iter(())
         starts = [next(starts_live) if s is not None else 0 for s in self.slots]
         entries = [Entry(s, [0], want=[0], key=k) for s, k in zip(self.slots, self.keys)]
-        for gid, _ in self.cache.kv_groups:
+        for gid, group in self.cache.paged_groups:
             for s in self.slots:
-                if s is not None and len(self.cache.page_list(gid, s)) > self.layout.table_widths[gid]:
+                if s is not None and group.table_entries(s) > self.layout.table_widths[gid]:
                     raise RuntimeError("the decode session was sized for fewer tokens")
         i = rec.turn % rec.RING
         if rec.staged_events[i] is not None:
@@ -192,12 +202,12 @@ class DecodeSession:
         for one position are the same bytes; fixed-size state is not, so it is put back,
         and so are the tokens the run drew."""
         keep_tokens = self.tokens.clone()
-        keep_state = [(g, g.data.clone()) for _, g in self.cache.state_groups]
+        put_back = self.cache.snapshots()
         self._run()
         torch.cuda.synchronize()
         self.tokens.copy_(keep_tokens)
-        for g, saved in keep_state:
-            g.data.copy_(saved)
+        for restore in put_back:
+            restore()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             self._run()

@@ -40,7 +40,8 @@ class Engine:
             max_sequences = pages                 # a live sequence holds at least one page
         self.cache = Cache(model.cache_needs(), model.cache_borrow(), max_tokens=max_tokens,
                            max_sequences=max_sequences, dtype=self.rt.dtype, device=self.rt.device)
-        self.uploader = BatchUploader(self.rt.device)
+        self.step_fields = tuple(model.step_fields())  # further fields of a step's description
+        self.uploader = BatchUploader(self.rt.device, self.step_fields)
         self.vocab_size = model.plan.vocab_size
         self.recorded_steps = RecordedSteps(self)      # HIP graphs of the one-token step
 

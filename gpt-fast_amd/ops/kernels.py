@@ -256,20 +256,32 @@ SPLIT_SAMPLING_ABOVE = 16384
 _split_workspaces = {}
 
 
+def _device_index(device) -> int:
+    dev = torch.device(device)
+    return torch.cuda.current_device() if dev.index is None else dev.index
+
+
 def _split_workspace(B: int, V: int, device) -> torch.Tensor:
     """The workspace of the many-workgroup sampler for this many rows: allocated and zeroed
-    once per device and size; the kernels leave its histograms zero again, so it is used call
-    after call (on one stream at a time) and recorded launches keep a valid address."""
-    key = (torch.device(device).index, B, V)
+    once per device, stream and size.  The kernels of a call leave its histograms zero again, so it is
+    used call after call and recorded launches keep a valid address; calls on different
+    streams get workspaces of their own, and a call whose launch failed drops its workspace
+    (its histograms may be left half counted)."""
+    key = (_device_index(device), torch.cuda.current_stream().cuda_stream
+           if not torch.cuda.is_current_stream_capturing() else "capture", B, V)
     ws = _split_workspaces.get(key)
+    if ws is None and key[1] == "capture":
+        # a recording replays on whatever stream; it uses the workspace its warm-up run made
+        for (dev, _, b, v), t in _split_workspaces.items():
+            if (dev, b, v) == (key[0], B, V):
+                return t
+        raise KernelError("the sampler's workspace must exist before a step is recorded: "
+                          "run the step once outside the recording")
     if ws is None:
-        if torch.cuda.is_current_stream_capturing():
-            raise KernelError("the sampler's workspace must exist before a step is recorded: "
-                              "run the step once outside the recording")
         lib = library("sampling")
         lib.gfa_sample_split_workspace.restype = ctypes.c_size_t
         n = lib.gfa_sample_split_workspace(_i(B), _i(V))
-        ws = torch.zeros(n // 4, dtype=torch.int32, device=device)
+        ws = torch.zeros(n // 4, dtype=torch.int32, device=torch.device("cuda", key[0]))
         _split_workspaces[key] = ws
     return ws
 
@@ -278,10 +290,14 @@ def _sample_split(logits, temperature, top_k, seed, seed_words, row_keys, positi
                   position_offset, out, probs):
     B, V = logits.shape
     ws = _split_workspace(B, V, logits.device)
-    check(library("sampling").gfa_sample_split(
+    code = library("sampling").gfa_sample_split(
         ptr(logits), _sz(logits.stride(0)), _i(B), _i(V), _f(temperature), _i(top_k),
         ctypes.c_uint64(seed & (2 ** 64 - 1)), ptr(seed_words), ptr(row_keys), ptr(positions),
-        _i(position_offset), ptr(out), ptr(probs), ptr(ws), stream_handle()), "sample_split")
+        _i(position_offset), ptr(out), ptr(probs), ptr(ws), stream_handle())
+    if code != 0:
+        for key in [k for k, t in _split_workspaces.items() if t is ws]:
+            del _split_workspaces[key]
+    check(code, "sample_split")
     return out
 
 

@@ -43,6 +43,24 @@ class Attention(Part):
     def replayable(self):
         return bool(getattr(self.position, "replayable", False))
 
+    def step_flops(self, q_lens, starts) -> float:
+        """Multiply-adds times two of a step that brings ``q_lens[b]`` tokens to sequences
+        that hold ``starts[b]``: the two projections, and scores and weighted sums over the
+        keys each token sees (a causal prompt counts its triangle, not the square)."""
+        s = self.spec
+        n = sum(q_lens)
+        flops = 2.0 * n * (self.wqkv_rows() + s.n_heads * s.head_dim) * s.dim
+        for q, start in zip(q_lens, starts):
+            keys = q * start + q * (q + 1) / 2.0
+            if s.window is not None:
+                keys = min(keys, q * float(s.window))
+            flops += 2.0 * 2.0 * s.n_heads * s.head_dim * keys
+        return flops
+
+    def wqkv_rows(self) -> int:
+        s = self.spec
+        return (s.n_heads + 2 * s.n_kv_heads) * s.head_dim
+
     prepares_norm = True
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 

@@ -72,6 +72,11 @@ class Part:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         pass
 
+    def step_fields(self):
+        """Further int32 fields of a step's description that this part reads
+        (``engine.batch.StepField``); none by default."""
+        return ()
+
 
 class _Registry:
     def __init__(self, what: str):

@@ -36,6 +36,17 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def step_flops(self, q_lens, starts) -> float:
+        """Matrix-product work of one run of this block (parts that do not say count as 0)."""
+        return sum(getattr(c, "step_flops", lambda q, s: 0.0)(q_lens, starts)
+                   for c in self.children().values())
+
+    def step_fields(self):
+        out = []
+        for child in self.children().values():
+            out += list(getattr(child, "step_fields", lambda: ())())
+        return out
+
     # Norm hand-over, optional for every part: a mixer or feed-forward that sets
     # ``prepares_norm`` takes ``then_norm=`` (the norm that reads the residual stream after
     # it) and ``takes_halves=`` (whether that norm's reader accepts an ops.linear.HalfNormed

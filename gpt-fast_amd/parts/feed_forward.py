@@ -30,6 +30,9 @@ class GatedFeedForward(Part):
     # at one row as the dot-product kernel that does not, and the norm kernel is saved)
     takes_prepared = 1
 
+    def step_flops(self, q_lens, starts) -> float:
+        return 2.0 * sum(q_lens) * 3 * self.spec.hidden * self.spec.dim
+
     def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
         return L.gated_into(x, self.w13, self.w2, residual, then_norm, takes_halves)
 

@@ -106,6 +106,26 @@ class DecoderModel:
     def cache_borrow(self) -> List[object]:
         return [run.cache_from for run in self.plan.order]
 
+    def step_flops(self, q_lens, starts, n_want: int) -> float:
+        """Matrix-product work (multiply-adds times two) of one step that brings
+        ``q_lens[b]`` tokens to sequences holding ``starts[b]`` and wants ``n_want`` rows of
+        logits: every run of the order, as its parts count themselves, and the head."""
+        flops = 2.0 * n_want * self.plan.dim * self.plan.vocab_size
+        for run in self.plan.order:
+            block = self.blocks[run.layer]
+            flops += getattr(block, "step_flops", lambda q, s: 0.0)(q_lens, starts)
+        return flops
+
+    def step_fields(self):
+        """The further fields of a step's description that the parts ask for, each once (by
+        name: layers of one kind ask for the same field)."""
+        seen = {}
+        parts = list(self.blocks) + [self.final_norm, self.input_position]
+        for part in parts:
+            for f in (getattr(part, "step_fields", lambda: ())() if part is not None else ()):
+                seen.setdefault(f.name, f)
+        return list(seen.values())
+
     # ------------------------------------------------------------------ step
     def forward(self, batch, cache) -> torch.Tensor:
         """float32 logits [n_wanted, vocab] of the step described by ``batch``."""

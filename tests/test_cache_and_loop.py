@@ -423,3 +423,84 @@ def test_cache_page_order_is_a_permutation():
     # a value tile: dims 16 j .. 16 j + 15, eight consecutive keys each: 16 bytes per dim, dims side by side
     assert [int(vp[16 + i, 40]) for i in range(16)] == list(range(int(vp[16, 40]), int(vp[16, 40]) + 128, 8))
     assert [int(vp[16, 40 + e]) for e in range(8)] == list(range(int(vp[16, 40]), int(vp[16, 40]) + 8))
+
+
+def test_a_cache_need_of_another_kind_and_values_of_another_width():
+    """Needs are an open table: a kind registered here gets a group of its class, takes part
+    in acquire / extend / release with the others, and can refuse a step as a whole.  Keys
+    and values of a KV need may have different widths."""
+    from dataclasses import dataclass
+
+    from gpt_fast_amd.cache.slots import CacheFull
+    from gpt_fast_amd.cache.store import Group, register_cache_need
+
+    @dataclass(frozen=True)
+    class BudgetNeed:
+        tokens: int
+
+    log = []
+
+    class BudgetGroup(Group):
+        """Takes at most ``need.tokens`` tokens per sequence."""
+
+        def __init__(self, need, entries, geometry, dtype, device):
+            self.need, self.entries, self.geometry = need, entries, geometry
+
+        def acquire(self, slot):
+            log.append(("acquire", slot))
+
+        def release(self, slot):
+            log.append(("release", slot))
+
+        def plan_extend(self, items, lengths):
+            for slot, n_new in items:
+                if lengths[slot] + n_new > self.need.tokens:
+                    raise CacheFull(f"slot {slot} would exceed {self.need.tokens} tokens")
+            return lambda: log.append(("extend", tuple(items)))
+
+    register_cache_need(BudgetNeed, BudgetGroup)
+    c = Cache([KVNeed(2, 8, None, value_dim=24), BudgetNeed(100), BudgetNeed(100), None],
+              [None, None, None, None], max_tokens=64 * 8, max_sequences=3,
+              dtype=torch.float32, device="cpu")
+    kv, budget = c.groups
+    assert isinstance(budget, BudgetGroup) and budget.entries == 2 and budget.geometry.n_slots == 3
+    assert kv.k.shape == (1, 9, 2, 64, 8) and kv.v.shape == (1, 9, 2, 24, 64)
+    assert kv.bytes_per_token() == 2 * (8 + 24) * 4
+    assert [g for _, g in c.paged_groups] == [kv]
+    a, b = c.acquire(), c.acquire()
+    c.extend_many([(a, 90), (b, 10)])
+    held = kv.pages.held
+    with pytest.raises(CacheFull, match="exceed 100"):
+        c.extend_many([(b, 70), (a, 11)])               # the budget refuses: nothing changes,
+    assert kv.pages.held == held and c.length(a) == 90 and c.length(b) == 10   # not even pages
+    c.extend_many([(b, 70)])
+    c.release(a)
+    c.release(b)
+    c.check()
+    assert [e[0] for e in log] == ["acquire", "acquire", "extend", "extend", "release", "release"]
+    with pytest.raises(TypeError, match="registered kind"):
+        Cache([object()], [None], max_tokens=64, max_sequences=1, dtype=torch.float32, device="cpu")
+
+
+def test_a_part_can_ask_for_a_field_of_its_own_in_the_steps_description():
+    """BatchLayout takes further fields; fill_host has each written by its own function, for
+    live rows and for rows that only fill a recorded batch's shape."""
+    from gpt_fast_amd.engine.batch import StepField
+
+    def fill(view, entries, starts, cache):
+        for b, (e, start) in enumerate(zip(entries, starts)):
+            view[b] = -1 if e.slot is None else start + len(e.tokens)
+
+    field = StepField("new_len", lambda n_tokens, n_seqs: n_seqs, fill)
+    c = Cache([KVNeed(1, 8)], [None], max_tokens=256, max_sequences=2, dtype=torch.float32, device="cpu")
+    a = c.acquire()
+    starts = c.extend_many([(a, 3)])
+    entries = [Entry(a, [1, 2, 3], want=[2]), Entry(None, [0], want=[0])]
+    lay = BatchLayout(4, 2, 2, {0: 2}, extra=[field])
+    host = np.zeros(lay.size, dtype=np.int32)
+    fill_host(lay, host, entries, [starts[0], 0], c)
+    off, count = lay.fields["new_len"]
+    assert count == 2 and list(host[off:off + 2]) == [3, -1]
+    assert off % 4 == 0 and lay.key() != BatchLayout(4, 2, 2, {0: 2}).key()
+    with pytest.raises(ValueError, match="tokens"):
+        BatchLayout(1, 1, 1, {}, extra=[StepField("tokens", lambda n, b: 1, fill)])

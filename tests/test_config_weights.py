@@ -373,6 +373,32 @@ def test_a_tokenizer_file_that_cannot_be_read_says_why(tmp_path):
         get_tokenizer(str(tmp_path))
 
 
+def test_sizes_and_work_of_a_step_come_from_the_architecture_and_the_parts():
+    """What a benchmark reports is asked of the architecture (flat sizes) and of the model's
+    parts (matrix-product work of a step), not read from one configuration class's fields.
+    The 8B shape's 2,048-token prompt by hand: linears, the causal triangle, one row of the
+    head (model.py:136-146, 191-227)."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.parts import Runtime
+    from gpt_fast_amd.parts.model import DecoderModel
+    arch, cfg = gfa.find_preset("llama-3.1-8b")
+    sizes = arch.describe(cfg)
+    assert sizes["n_layer"] == 32 and sizes["dim"] == 4096 and sizes["n_kv_heads"] == 8
+    assert sizes["intermediate_size"] == 14336 and sizes["vocab_size"] == 128256
+    assert sizes["rope_scaling"].startswith("llama3 factor 8") and len(sizes) <= 12
+    assert all(isinstance(v, (int, float, str)) for v in sizes.values())
+    model = DecoderModel(arch.plan(cfg), Runtime(torch.bfloat16, "cpu"))
+    D, H, G, hd, I, V, L, T = 4096, 32, 8, 128, 14336, 128256, 32, 2048
+    linears = 2.0 * T * L * ((H + 2 * G) * hd * D + H * hd * D + 3 * I * D)
+    triangle = L * 2.0 * 2.0 * H * hd * (T * (T + 1) / 2)
+    assert model.step_flops([T], [0], n_want=1) == linears + triangle + 2.0 * D * V
+    # a one-token step at position 100 for each of three sequences
+    one = model.step_flops([1, 1, 1], [100, 100, 100], n_want=3)
+    assert one == 3 * (linears / T + L * 4.0 * H * hd * 101 + 2.0 * D * V)
+    raw = arch.config_dict(cfg)
+    assert raw[arch.layer_count_key] == 32
+
+
 def test_a_library_is_rebuilt_when_its_source_changes(tmp_path, monkeypatch):
     """The stamp beside a built library holds a hash of source, common header and flags; a
     library whose stamp does not fit is not current."""

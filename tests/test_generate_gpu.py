@@ -596,6 +596,22 @@ def test_command_line_random_weights_and_a_batch(tmp_path):
     assert "Prompt Length: 4" in proc.stdout
 
 
+def test_command_line_profile_writes_a_trace_of_the_last_sample(tmp_path):
+    """--profile PATH (generate.py:380-385, 403-407): the last sample runs under the profiler
+    and its trace is written to PATH.json; the trace names kernels of this library."""
+    import json as _json
+    trace = tmp_path / "trace"
+    proc = _cli("--random", "tiny-llama-a", "--prompt", 6, "--num_samples", 2, "--max_new_tokens", 4,
+                "--temperature", 0, "--profile", trace, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    path = tmp_path / "trace.json"
+    assert path.is_file() and path.stat().st_size > 1000
+    events = _json.loads(path.read_text())["traceEvents"]
+    names = {e.get("name", "") for e in events}
+    assert any("kernel" in n and ("skinny" in n or "attention" in n or "rmsnorm" in n or "embed" in n)
+               for n in names), sorted(names)[:40]
+
+
 def test_command_line_refusals(tmp_path_factory):
     folder = util.make_folder(tmp_path_factory.getbasetemp(), "A")
     for args, needle in (

@@ -412,6 +412,147 @@ def test_toy_mixer_with_state_through_generate(on_device):
             assert float(row[tok]) >= float(row.max()) - 1e-4 * float(row.abs().max()), (i, tok)
 
 
+# --------------------------------------------------------------------------------------
+# A mixer whose cache is of a kind of its own - a ring of its last SIZE inputs per sequence,
+# registered from here with the class that stores it - and which asks for a field of its own
+# in every step's description: the ring slot each token writes to.
+@dataclasses.dataclass(frozen=True)
+class RecentMeanSpec:
+    dim: int
+    size: int
+    kind: str = "toy_recent_mean"
+
+
+@dataclasses.dataclass(frozen=True)
+class RingNeed:
+    dim: int
+    size: int
+
+
+def _recent_mean_classes():
+    from gpt_fast_amd.cache.store import Group, register_cache_need
+    from gpt_fast_amd.engine.batch import StepField
+    from gpt_fast_amd.parts import Param, Part
+
+    class RingGroup(Group):
+        """[entries, slots + 1, size + 1, dim]: the ring, and a row whose first element counts
+        the inputs seen; the last slot belongs to no sequence."""
+
+        def __init__(self, need, entries, geometry, dtype, device):
+            self.need = need
+            self.data = torch.zeros((entries, geometry.n_slots + 1, need.size + 1, need.dim),
+                                    dtype=torch.float32, device=device)
+            self.acquired = 0
+
+        def acquire(self, slot):
+            self.data[:, slot].zero_()
+            self.acquired += 1
+
+        def snapshot(self):
+            saved = self.data.clone()
+            return lambda: self.data.copy_(saved)
+
+    register_cache_need(RingNeed, RingGroup)
+
+    class RecentMean(Part):
+        """residual += mix(mean of the last ``size`` normed inputs, this token's included)."""
+
+        def __init__(self, spec, rt):
+            self.spec = spec
+
+        def parameters(self):
+            return {"mix": Param((self.spec.dim, self.spec.dim))}
+
+        def bind(self, tensors):
+            self.mix = tensors["mix"]
+
+        def cache_need(self):
+            return RingNeed(self.spec.dim, self.spec.size)
+
+        def step_fields(self):
+            size = self.spec.size
+
+            def fill(view, entries, starts, cache):
+                n = 0
+                for e, start in zip(entries, starts):
+                    for i in range(len(e.tokens)):
+                        view[n] = (start + i) % size
+                        n += 1
+            return [StepField("ring_slot", lambda n_tokens, n_seqs: n_tokens, fill)]
+
+        def forward(self, x, batch, entry, residual):
+            ring = entry.group.data[entry.index]                  # [slots + 1, size + 1, dim]
+            q_start = batch.host_field("q_start")
+            slots = batch.host_field("slots")
+            ring_slot = batch.ring_slot.long()                    # the field, on the device
+            for b in range(batch.n_seqs):
+                r = ring[int(slots[b])]
+                for n in range(int(q_start[b]), int(q_start[b + 1])):
+                    r[ring_slot[n]] = x[n].float()
+                    r[-1, 0] += 1
+                    count = torch.clamp(r[-1, 0], max=self.spec.size)
+                    residual[n] += (r[:-1].sum(0) / count) @ self.mix.float().T
+
+    return RingGroup, RecentMean
+
+
+def test_toy_mixer_with_a_cache_kind_and_a_step_field_of_its_own():
+    """Neither the cache nor the step's description has to change for a mixer that needs
+    another kind of storage and another per-step field: both are registered from here.
+    Compared with the plain computation (a windowed mean over the whole sequence), whole and
+    cut into steps beside another sequence, and through generate()."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.config.spec import LayerSpec, ModelPlan, NormSpec, Run
+    from gpt_fast_amd.parts import Runtime, register_mixer
+    from gpt_fast_amd.parts.model import DecoderModel
+    RingGroup, RecentMean = _recent_mean_classes()
+    register_mixer("toy_recent_mean", RecentMean)
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_A)
+    base = arch.plan(cfg)
+    D, SIZE = cfg.hidden_size, 5
+    toy = LayerSpec(name="toy", mixer=RecentMeanSpec(D, SIZE), mixer_norm=NormSpec(D, 1e-5),
+                    feed_forward=base.layers[0].feed_forward, feed_forward_norm=NormSpec(D, 1e-5))
+    plan = ModelPlan(dim=D, vocab_size=cfg.vocab_size, layers=[base.layers[0], toy],
+                     order=[Run(0), Run(1), Run(1)], final_norm=base.final_norm, max_positions=4096)
+    model = DecoderModel(plan, Runtime(torch.float32, DEV))
+    assert [f.name for f in model.step_fields()] == ["ring_slot"]      # asked for twice, kept once
+    w = _random_parameters(model, 41)
+    eng = gfa.Engine.from_plan(plan, {k: v.to(DEV) for k, v in w.items()}, "float32", DEV,
+                               max_tokens=1024, max_sequences=4)
+    ring_groups = [g for g in eng.cache.groups if isinstance(g, RingGroup)]
+    assert len(ring_groups) == 1 and ring_groups[0].data.shape[:2] == (2, 5)   # two runs, 4 + 1 slots
+    pcfg = plain.config_from_dict(util.TINY_A)
+
+    def plain_logits(toks):
+        def toy_block(x):
+            xn = plain.rms_norm(x, w["toy.mixer_norm.weight"], 1e-5)
+            mean = torch.stack([xn[max(0, t - SIZE + 1):t + 1].mean(0) for t in range(x.shape[0])])
+            x = x + mean @ w["toy.mixer.mix"].T
+            hn = plain.rms_norm(x, w["toy.feed_forward_norm.weight"], 1e-5)
+            w13 = w["toy.feed_forward.w13"]
+            I = w13.shape[0] // 2
+            return x + plain.feed_forward(hn, w13[:I], w13[I:], w["toy.feed_forward.w2"])
+        x = w["tok_embeddings.weight"][torch.tensor(toks)]
+        x = _plain_dense_ffn(_plain_attention_block(x, w, "layers.0.", pcfg), w, "layers.0.", pcfg)
+        x = toy_block(toy_block(x))
+        return plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
+
+    V = cfg.vocab_size
+    toks = util.random_tokens(V, 40, 9)
+    want = plain_logits(toks)
+    _steps_equal_whole(eng, toks, want, V, TOL_F32)
+    _steps_equal_whole(eng, toks, want, V, TOL_F32)              # rings of used slots start empty
+    prompts = [util.random_tokens(V, n, 500 + n) for n in (3, 11)]
+    out = gfa.generate(eng, prompts, max_new_tokens=8, temperature=0.0).tokens
+    for p, new in zip(prompts, out):
+        logits = plain_logits(p + new)
+        for i, tok in enumerate(new):
+            row = logits[len(p) - 1 + i]
+            assert float(row[tok]) >= float(row.max()) - 1e-4 * float(row.abs().max())
+    assert eng.cache.slots.held == 0
+
+
 def test_plan_level_steps_scale_position_and_cap():
     """What a plan may state around its layers, none of which Llama uses: a factor on the
     embedded rows, a position encoding added to them (a toy table of learned vectors,

@@ -218,7 +218,7 @@ def main():
             "model": args.preset, **sizes, "n_layer_full": full_layers,
             "global_batch": batch, "seq_len": context,
             "prompt_len": args.prompt_lens or args.prompt_len,
-            "new_tokens": args.warmup + args.steps,
+            "new_tokens": args.warmup + runs * args.steps,
             "weights": "random N(0,0.02) bf16", "sampling": "greedy", "hip_graph": use_graph,
             "parallelism": "single GPU",
         },

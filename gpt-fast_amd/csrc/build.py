@@ -17,7 +17,8 @@ import threading
 import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-MODULES = ("core", "sampling", "gemm_bf16", "gemm_wide_bf16", "attention_bf16", "ceilings")
+MODULES = ("core", "sampling", "gemm_bf16", "gemm_wide_bf16", "gemm_tiled_bf16", "attention_bf16",
+           "ceilings")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

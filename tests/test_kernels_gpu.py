@@ -141,6 +141,54 @@ def test_products_of_up_to_64_rows(M, N, K_):
         close(W.product_gated(x, w), (a * torch.sigmoid(a)) * ref[:, I:], 1e-2)
 
 
+def _tiled_by_hand(w, gate):
+    """The tiled form written from its description: [tiles][Kp / 8][16][8], Kp = K rounded up to
+    128, zeros beyond the matrix; gate: tile t = rows 8 t .. + 7 of W1, then the same rows of W3."""
+    rows, K = w.shape
+    Kp = (K + 127) // 128 * 128
+    if gate:
+        I = rows // 2
+        tiles = (I + 7) // 8
+        src = torch.zeros(tiles, 16, Kp, dtype=w.dtype)
+        for t in range(tiles):
+            n = min(8, I - 8 * t)
+            src[t, :n, :K] = w[8 * t:8 * t + n]
+            src[t, 8:8 + n, :K] = w[I + 8 * t:I + 8 * t + n]
+    else:
+        tiles = (rows + 15) // 16
+        src = torch.zeros(tiles * 16, Kp, dtype=w.dtype)
+        src[:rows, :K] = w
+        src = src.view(tiles, 16, Kp)
+    return src.view(tiles, 16, Kp // 8, 8).permute(0, 2, 1, 3).contiguous().view(-1)
+
+
+@pytest.mark.parametrize("M", [17, 25, 32, 33, 48, 64, 3])
+@pytest.mark.parametrize("N,K_", [(40, 64), (136, 200), (1000, 328), (256, 4096), (77, 72), (4096, 1024),
+                                  (6144, 512), (2000, 1536)])
+def test_products_over_weights_in_operand_order(M, N, K_):
+    """The 17..64-row kernels that read W in the matrix cores' operand order: the tiled copy
+    itself, the partial sums of a sliced product (added in slice order), the one-kernel float
+    product, and the gate with its eight-and-eight tiles - at widths and inner sizes that are
+    no multiples of the tile (16 rows of W, 128 values of k), against float64."""
+    from gpt_fast_amd.ops import gemm_tiled_bf16 as T
+    torch.manual_seed(M + N)
+    x = bf(torch.randn(M, K_))
+    w = bf(torch.randn(N, K_) / math.sqrt(K_))
+    ref = x.double() @ w.double().T
+    t = T.tile(w.to(DEV))
+    assert torch.equal(t.data.cpu(), _tiled_by_hand(w, False))
+    part = T.partial_sums(x.to(DEV), t)
+    assert part.shape[1:] == (M, N) and part.shape[0] == T.slices(N, K_)
+    close(part.sum(0), ref, 1e-5)
+    close(T.product_f32(x.to(DEV), t), ref, 1e-5)
+    if N % 2 == 0:
+        I = N // 2
+        tg = T.tile(w.to(DEV), gate=True)
+        assert torch.equal(tg.data.cpu(), _tiled_by_hand(w, True))
+        a, b = ref[:, :I], ref[:, I:]
+        close(T.product_gated(x.to(DEV), tg), a * torch.sigmoid(a) * b, 1.5e-2)
+
+
 def test_sliced_product_equals_its_slices_added_in_order():
     from gpt_fast_amd.ops import gemm_wide_bf16 as W
     torch.manual_seed(15)

@@ -381,6 +381,84 @@ __global__ __launch_bounds__(256) void rope_cache_bf16x8_kernel(
     }
 }
 
+// The same with the rows given as float partial sums of a sliced product, part [S, N, width]:
+// the slices are added in order (the sum a kernel of its own would form), rotated and stored,
+// so that the product's second kernel is this one.  The rotation then works on the float sums
+// instead of their bfloat16 rounding.
+__global__ __launch_bounds__(256) void rope_cache_sliced_bf16x8_kernel(
+        const float* __restrict__ part, int S, size_t slice, bf16_t* __restrict__ q_out,
+        bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const float* __restrict__ freqs,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, int table_stride, int H, int Hkv, int hd, int rot) {
+    const int n = blockIdx.x;
+    const int per_head = hd / 8;
+    const int qk_chunks = (H + Hkv) * per_head, v_chunks = Hkv * per_head;
+    const int pos = tok_pos[n];
+    extern __shared__ float cs[];                          // [rot / 2][2]
+    if (blockIdx.y * 256 < qk_chunks) {
+        for (int i = threadIdx.x; i < rot / 2; i += 256)
+            sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
+        __syncthreads();
+    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= qk_chunks + v_chunks) return;
+    const int head = c / per_head, d0 = (c - head * per_head) * 8;
+    const float* src = part + ((size_t)n * (H + 2 * Hkv) + head) * hd + d0;
+    float v[8];
+    {
+        const float4 a = *(const float4*)src, b = *(const float4*)(src + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+    for (int s = 1; s < S; ++s) {
+        const float4 a = *(const float4*)(src + s * slice), b = *(const float4*)(src + s * slice + 4);
+        v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+    }
+    int page = 0;
+    if (k_pages && head >= H) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+    const int off = pos % GFA_PAGE;
+    union { uint4 u; bf16_t e[8]; } out;
+    if (head < H + Hkv) {
+        if (d0 < rot) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const float a = v[2 * p], b = v[2 * p + 1];
+                const float c_ = cs[d0 + 2 * p], s_ = cs[d0 + 2 * p + 1];
+                out.e[2 * p] = float_to_bf16(a * c_ - b * s_);
+                out.e[2 * p + 1] = float_to_bf16(b * c_ + a * s_);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) out.e[j] = float_to_bf16(v[j]);
+        }
+        if (head < H) {
+            *(uint4*)(q_out + ((size_t)n * H + head) * hd + d0) = out.u;
+        } else if (k_pages) {
+            *(uint4*)(k_pages + key_elem(page, head - H, off, d0, Hkv, hd)) = out.u;
+        }
+    } else if (v_pages) {
+        const int g = head - H - Hkv;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v_pages[value_elem(page, g, d0 + j, off, Hkv, hd)] = float_to_bf16(v[j]);
+    }
+}
+
+// part [S, n_tokens, (H + 2 Hkv) * hd] float; interleaved pairs, hd and rot multiples of 8.
+extern "C" int gfa_rope_cache_write_sliced(const float* part, int S, void* q_out, void* k_pages,
+                                           void* v_pages, const float* freqs, const int* tok_seq,
+                                           const int* tok_pos, const int* table, int table_stride,
+                                           int n_tokens, int H, int Hkv, int hd, int rot,
+                                           hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (S <= 0 || hd % 8 != 0 || rot % 8 != 0 || rot > hd || (rot > 0 && !freqs))
+        return (int)hipErrorInvalidValue;
+    const dim3 grid(n_tokens, ((H + 2 * Hkv) * (hd / 8) + 255) / 256);
+    const size_t slice = (size_t)n_tokens * (H + 2 * Hkv) * hd;
+    rope_cache_sliced_bf16x8_kernel<<<grid, 256, (size_t)(rot > 0 ? rot : 2) * sizeof(float), stream>>>(
+        part, S, slice, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, freqs, tok_seq, tok_pos,
+        table, table_stride, H, Hkv, hd, rot);
+    return GFA_LAUNCH_RESULT();
+}
+
 extern "C" int gfa_rope_cache_write(const void* qkv, void* q_out, void* k_pages, void* v_pages,
                                     const float* freqs, const int* tok_seq, const int* tok_pos,
                                     const int* table, int table_stride, int n_tokens, int H,

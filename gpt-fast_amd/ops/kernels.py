@@ -167,6 +167,40 @@ def rope_cache_write(qkv: torch.Tensor, freqs: Optional[torch.Tensor], tok_seq, 
     return q_out
 
 
+def rope_cache_write_sliced(part: torch.Tensor, freqs: Optional[torch.Tensor], tok_seq, tok_pos, table,
+                            k_pages, v_pages, n_heads: int, n_kv_heads: int, head_dim: int,
+                            rotary_dim: int):
+    """:func:`rope_cache_write` for rows given as the float partial sums of a sliced product,
+    part [S, N, (H+2G)*hd]: slices added in order, pairs (2i, 2i+1) rotated, bfloat16 q
+    returned and k, v stored.  head_dim and rotary_dim multiples of 8."""
+    require_device(part, freqs, tok_seq, tok_pos, table, k_pages, v_pages)
+    require_contiguous(part=part, freqs=freqs, tok_seq=tok_seq, tok_pos=tok_pos, table=table)
+    _want(part, torch.float32, "part")
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if part.dim() != 3 or part.shape[2] != width:
+        raise KernelError(f"rope: the partial sums are {tuple(part.shape)}, expected [S, N, {width}]")
+    S, n, _ = part.shape
+    if head_dim % 8 or rotary_dim % 8 or not 0 <= rotary_dim <= head_dim:
+        raise KernelError("rope over partial sums: head_dim and rotary_dim in multiples of 8")
+    if rotary_dim:
+        _want(freqs, torch.float32, "freqs")
+        if freqs.numel() != rotary_dim // 2:
+            raise KernelError(f"rope: {freqs.numel()} frequencies for rotary_dim {rotary_dim}")
+    if tok_seq.numel() < n or tok_pos.numel() < n:
+        raise KernelError("rope: token maps are shorter than the batch")
+    for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos), ("table", table)):
+        _want(t, torch.int32, name)
+    if (k_pages is None) != (v_pages is None):
+        raise KernelError("rope: give both k_pages and v_pages, or neither")
+    _check_pages(k_pages, v_pages, n_kv_heads, head_dim, torch.bfloat16)
+    q_out = torch.empty((n, n_heads, head_dim), dtype=torch.bfloat16, device=part.device)
+    check(library("core").gfa_rope_cache_write_sliced(
+        ptr(part), _i(S), ptr(q_out), ptr(k_pages), ptr(v_pages), ptr(freqs), ptr(tok_seq),
+        ptr(tok_pos), ptr(table), _i(table.shape[1]), _i(n), _i(n_heads), _i(n_kv_heads),
+        _i(head_dim), _i(rotary_dim), stream_handle()), "rope_cache_write_sliced")
+    return q_out
+
+
 # ----------------------------------------------------------------------------- attention
 def attention_generic(q: torch.Tensor, k_pages, v_pages, tok_seq, tok_pos, table,
                       scale: float, window: int = 0, out: Optional[torch.Tensor] = None):

@@ -59,8 +59,9 @@ def _fast():
 # matrix cores' operand order (gemm_tiled_bf16), if the device has room for that copy: measured
 # on the 8B shapes at 17..64 rows, 41-44 us against 55-65 for the gate product with the vendor
 # library and the gate kernel behind it, 22-24 against 29-39 for the second feed-forward product,
-# 11-13 against 13-18 for the projections.  Below it, the chain of few-row kernels is used.
-TILED_FROM_ROWS = 25
+# 11-13 against 13-18 for the projections; per step 3.60-3.65 ms at 17..24 rows against
+# 4.01-4.07 for the chain of few-row kernels, which is what runs there without the copy.
+TILED_FROM_ROWS = 17
 
 
 def _tiled_for(rows: int, w: torch.Tensor, gate: bool = False):
@@ -95,8 +96,29 @@ class HalfNormed:
         return self.xg.dtype
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
-    """[M, N] = x [M, K] times w [N, K] transposed, in ``out_dtype`` (default: x's)."""
+class SlicedRows:
+    """Rows of a product whose inner size was cut into slices, before the slices are added:
+    ``part`` float32 [S, M, N].  A reader that adds them on its way (the rotation and cache
+    write of ``ops.kernels.rope_cache_write_sliced``) saves the pass that :meth:`rows` is."""
+
+    __slots__ = ("part", "dtype")
+
+    def __init__(self, part, dtype):
+        self.part, self.dtype = part, dtype
+
+    @property
+    def shape(self):
+        return tuple(self.part.shape[1:])
+
+    def rows(self) -> torch.Tensor:
+        """[M, N] in the product's type: the slices added in order."""
+        return _wide().sum_store(self.part, self.dtype)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           may_stay_sliced: bool = False):
+    """[M, N] = x [M, K] times w [N, K] transposed, in ``out_dtype`` (default: x's).
+    ``may_stay_sliced``: the caller also takes a :class:`SlicedRows`."""
     out_dtype = out_dtype or x.dtype
     if isinstance(x, HalfNormed):
         return _fast().skinny_after_chain(x.xg, x.ssq, x.eps, w, out_dtype=out_dtype)
@@ -112,7 +134,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         from . import gemm_tiled_bf16 as T
         if out_dtype == torch.float32:
             return T.product_f32(x, t)
-        return _wide().sum_store(T.partial_sums(x, t), out_dtype)
+        rows = SlicedRows(T.partial_sums(x, t), out_dtype)
+        return rows if may_stay_sliced else rows.rows()
     if out_dtype == torch.float32:
         return _fast().wide_f32_out(x, w)
     return torch.matmul(x, w.t())
@@ -156,7 +179,8 @@ def _chains(rows: int, dtype, w, then_norm, takes_halves: bool) -> bool:
     ``then_norm`` for a reader that takes it in halves."""
     return (takes_halves and dtype == torch.bfloat16
             and getattr(then_norm, "row_and_column_form", None) is not None
-            and _fast().can_chain_norm(rows, w.shape[0], w.shape[1]))
+            and _fast().can_chain_norm(rows, w.shape[0], w.shape[1])
+            and _tiled_for(rows, w) is None)        # with the second copy, 17..24 rows go there
 
 
 def _wide():

@@ -72,7 +72,8 @@ class Attention(Part):
             # few rows: projection, rotation and cache write in one kernel
             q = fused(x, self.wqkv, batch, entry, s.n_heads, s.n_kv_heads, s.head_dim)
         if q is None:
-            qkv = L.linear(x, self.wqkv)                                    # model.py:195
+            qkv = L.linear(x, self.wqkv,                                    # model.py:195
+                           may_stay_sliced=getattr(self.position, "takes_sliced", False))
             q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
                                                s.head_dim)                  # model.py:201-207
         # the output projection may take the heads' results in the order it loads them in

@@ -63,14 +63,23 @@ class RotaryPosition(Part):
         self.freqs_host = freqs.to(torch.float32)
         self.freqs = self.freqs_host.to(runtime.device)
 
+    # qkv may come as ops.linear.SlicedRows (a sliced product's partial sums): they are added
+    # on the way where the kernel for that fits
+    takes_sliced = True
+
     def rotate_and_store(self, qkv, batch, entry, n_heads, n_kv_heads, head_dim):
         write = entry is not None and entry.writes
+        pages = (entry.k_pages if write else None, entry.v_pages if write else None)
+        if isinstance(qkv, L.SlicedRows):
+            if (self.spec.layout == "interleaved" and qkv.dtype == torch.bfloat16
+                    and head_dim % 8 == 0 and self.spec.rotary_dim % 8 == 0):
+                return K.rope_cache_write_sliced(
+                    qkv.part, self.freqs, batch.tok_seq, batch.tok_pos, batch.table(entry.group_id),
+                    *pages, n_heads, n_kv_heads, head_dim, self.spec.rotary_dim)
+            qkv = qkv.rows()
         return K.rope_cache_write(
-            qkv, self.freqs, batch.tok_seq, batch.tok_pos, batch.table(entry.group_id),
-            entry.k_pages if write else None, entry.v_pages if write else None,
-            n_heads, n_kv_heads, head_dim, self.spec.rotary_dim,
-            self.LAYOUTS[self.spec.layout])
-
+            qkv, self.freqs, batch.tok_seq, batch.tok_pos, batch.table(entry.group_id), *pages,
+            n_heads, n_kv_heads, head_dim, self.spec.rotary_dim, self.LAYOUTS[self.spec.layout])
 
     def project_rotate_store(self, x, wqkv, batch, entry, n_heads, n_kv_heads, head_dim):
         """Projection + rotation + cache write in one kernel for few rows (interleaved

@@ -111,6 +111,42 @@ def early_uses(items, wait_states: int = WAIT_STATES):
     return bad
 
 
+def loads_touched_before_their_wait(assembly: str):
+    """Loads that a kernel writes as inline asm are not known to the compiler as loads: it may
+    use their registers as soon as the statement is over, while the data is still under way.
+    The kernels therefore name those registers in the asm wait that follows (which orders
+    every reader behind it).  This checks the result: between an asm ``global_load`` and the
+    next asm ``s_waitcnt vmcnt`` in the kernel's text, no instruction may mention the load's
+    registers.  Returns [(kernel, load, offending instruction)]."""
+    out = []
+    for chunk in re.split(r"\n(?=[A-Za-z_]\w*:)", assembly):
+        m = re.match(r"([A-Za-z_]\w*):", chunk)
+        if not m:
+            continue
+        lines = chunk.split("\n")
+        for i, line in enumerate(lines):
+            if "#ASMSTART" not in line or i + 1 >= len(lines) or "global_load" not in lines[i + 1]:
+                continue
+            load = lines[i + 1].strip()
+            dst = registers(load.split(None, 1)[1].split(",")[0])
+            j = i + 3                                      # behind the load's #ASMEND
+            while j < len(lines):
+                t = lines[j].split(";")[0].strip() if "#ASM" not in lines[j] else lines[j].strip()
+                if "#ASMSTART" in t and j + 1 < len(lines) and "s_waitcnt" in lines[j + 1] \
+                        and "vmcnt" in lines[j + 1]:
+                    break
+                if t.startswith("s_endpgm"):
+                    out.append((m.group(1), load, "the kernel ends before a wait"))
+                    break
+                if t and not t.startswith(".") and "#ASM" not in t:
+                    operands = t.split(None, 1)[1] if len(t.split(None, 1)) > 1 else ""
+                    if registers(operands) & dst:
+                        out.append((m.group(1), load, t))
+                        break
+                j += 1
+    return out
+
+
 def assembly_of(module: str) -> str:
     """The device assembly of csrc/<module>.hip with the library's own flags, compiled once
     per state of the sources into the temporary directory."""

@@ -62,7 +62,7 @@ _Z2okv:
     assert len(isa_scan.early_uses(isa_scan.kernels_of(early)["_Z2okv"])) == 1
 
 
-MODULES = ("attention_bf16", "gemm_bf16", "gemm_wide_bf16", "ceilings")
+MODULES = ("attention_bf16", "gemm_bf16", "gemm_wide_bf16", "gemm_tiled_bf16", "ceilings")
 
 
 @pytest.fixture(scope="module")
@@ -80,3 +80,26 @@ def test_no_kernel_uses_a_matrix_result_too_early(assemblies, module):
     bad = {k: isa_scan.early_uses(kernels[k]) for k in with_matrix}
     bad = {k: v for k, v in bad.items() if v}
     assert not bad, bad
+
+
+def test_registers_of_hand_written_loads_wait_for_their_data(assemblies):
+    """gemm_tiled_bf16 requests x by asm loads; nothing may touch their registers before the
+    asm wait that names them.  The reader is checked on a sequence that does."""
+    touched = """
+tiled:
+	;;#ASMSTART
+	global_load_dwordx4 v[72:75], v[2:3], off
+	;;#ASMEND
+	v_cndmask_b32_e64 v75, 0, v75, s[4:5]
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	s_endpgm
+"""
+    found = isa_scan.loads_touched_before_their_wait(touched)
+    assert len(found) == 1 and "v_cndmask" in found[0][2]
+    assert isa_scan.loads_touched_before_their_wait(touched.replace("v75, 0, v75", "v80, 0, v81")) == []
+    text = assemblies["gemm_tiled_bf16"]
+    assert text.count("global_load_dwordx4") > text.count(" nt") > 0       # asm loads are there
+    assert "#ASMSTART" in text
+    assert isa_scan.loads_touched_before_their_wait(text) == []

@@ -630,6 +630,39 @@ def test_rope_and_cache_write(dtype, layout, H, G, hd, rot):
     assert torch.equal(q2.reshape(N, -1), qkv[:, :H * hd])
 
 
+@pytest.mark.parametrize("H,G,hd,rot,S", [(4, 2, 16, 16, 3), (3, 1, 48, 32, 1), (32, 8, 128, 128, 4), (2, 2, 32, 0, 5)])
+def test_rope_and_cache_write_over_partial_sums(H, G, hd, rot, S):
+    """The rotation and cache write that adds a sliced product's partial sums on its way:
+    float partial sums [S, N, width] in, bfloat16 q and pages out, against float64 of the
+    summed rows."""
+    torch.manual_seed(16)
+    pos = [0, 1, 63, 64, 130, 4000]
+    N = len(pos)
+    part = torch.randn(S, N, (H + 2 * G) * hd)
+    freqs = 1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / max(rot, 1)))
+    table = torch.tensor([[5, 3, 0, 1] + [2] * 60], dtype=torch.int32)
+    kp = torch.zeros(6, G, 64, hd, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(6, G, hd, 64, dtype=torch.bfloat16, device=DEV)
+    q_out = K().rope_cache_write_sliced(
+        part.to(DEV), freqs.to(DEV) if rot else None, torch.zeros(N, dtype=torch.int32, device=DEV),
+        torch.tensor(pos, dtype=torch.int32, device=DEV), table.to(DEV), kp, vp, H, G, hd, rot).cpu()
+    assert q_out.dtype == torch.bfloat16 and q_out.shape == (N, H, hd)
+    x = part.double().sum(0).reshape(N, H + 2 * G, hd)
+    ref = x.clone()
+    if rot:
+        ang = torch.tensor(pos, dtype=torch.float32)[:, None] * freqs[None, :]
+        c, s = torch.cos(ang.double())[:, None, :], torch.sin(ang.double())[:, None, :]
+        a, b = x[:, :H + G, 0:rot:2], x[:, :H + G, 1:rot:2]
+        ref[:, :H + G, 0:rot:2] = a * c - b * s
+        ref[:, :H + G, 1:rot:2] = b * c + a * s
+    close(q_out, ref[:, :H], 1e-2)
+    kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
+    for n, p in enumerate(pos):
+        page = int(table[0, p // 64])
+        close(kc[page, :, p % 64], ref[n, H:H + G], 1e-2)
+        close(vc[page, :, :, p % 64], ref[n, H + G:], 1e-2)
+
+
 def test_argmax_and_sampling():
     from gpt_fast_amd.sampling import SamplingParams, logits_to_probs, sample
     import plain_llama as plain

@@ -386,7 +386,15 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     constexpr int HDM = DS * 32;                          // head size the tiles are laid out for
     constexpr int KBYTES = 64 * HDM * 2, VBYTES = HDM * 64 * 2;   // a page's keys, its values
     constexpr int K_PER = KBYTES / 16 / 256, V_PER = VBYTES / 16 / 256;   // copies per thread
-    extern __shared__ __attribute__((aligned(16))) char smem[];   // 2 K tiles, then 2 V tiles
+    // Two pages of keys and two of values, each an LDS object of its own: the compiler then
+    // knows that a copy into one of them (global_load_lds) cannot change what the operand reads
+    // take from the other, and does not make those reads wait for the copy.  With one array
+    // indexed by the page's parity it put a wait for all copies in front of every page's
+    // products, so that no copy overlapped the arithmetic of its own wave.
+    __shared__ __attribute__((aligned(16))) char kb0[KBYTES];
+    __shared__ __attribute__((aligned(16))) char kb1[KBYTES];
+    __shared__ __attribute__((aligned(16))) char vb0[VBYTES];
+    __shared__ __attribute__((aligned(16))) char vb1[VBYTES];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int seq = blockIdx.z;
@@ -458,9 +466,9 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     // lanes (keys) or 1 KB per wave (values): no two lanes of a pass share a bank.
     const int hdr = FULL ? HDM : hd;
     const int page_slots = 8 * hdr;                        // 16-byte slots of keys (of values) per page
-    auto copy_keys = [&](int pg) {
+    auto copy_keys = [&](int pg, char* kbuf) {
         const char* src = (const char*)(k_pages + cache_region(pages[pg], g, Hkv, hd)) + threadIdx.x * 16;
-        char* dst = smem + (pg & 1) * KBYTES + wave * 1024;
+        char* dst = kbuf + wave * 1024;
 #pragma unroll
         for (int i = 0; i < K_PER; ++i)
             if (FULL || (int)threadIdx.x + i * 256 < page_slots)
@@ -468,9 +476,9 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
                     (const __attribute__((address_space(1))) void*)(src + i * 4096),
                     (__attribute__((address_space(3))) void*)(dst + i * 4096), 16, 0, 0);
     };
-    auto copy_values = [&](int pg) {
+    auto copy_values = [&](int pg, char* vbuf) {
         const char* src = (const char*)(v_pages + cache_region(pages[pg], g, Hkv, hd)) + threadIdx.x * 16;
-        char* dst = smem + 2 * KBYTES + (pg & 1) * VBYTES + wave * 1024;
+        char* dst = vbuf + wave * 1024;
 #pragma unroll
         for (int i = 0; i < V_PER; ++i)
             if (FULL || (int)threadIdx.x + i * 256 < page_slots)
@@ -482,12 +490,11 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     // newest key hold no data yet (whatever the cache held before): their values are set to
     // zero, by the thread that copied them, so that probability 0 times them is 0.  Value slot
     // s holds keys 32 (s / 64 % 2) + 8 (s / 16 % 4) .. + 7.
-    auto copies_landed = [&](int v_pg) {
+    auto copies_landed = [&](int v_pg, char* vt) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (v_pg > page_hi) return;
         const int keys_ok = wg_pmax - v_pg * 64;
         if (keys_ok >= 63) return;
-        char* vt = smem + 2 * KBYTES + (v_pg & 1) * VBYTES;
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
             const int slot = threadIdx.x + i * 256;
@@ -513,9 +520,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
     // the second product.  The wave's priority is raised while it issues matrix instructions,
     // so that the other waves of the SIMD fill the gaps with their vector work and not the
     // other way round.
-    auto compute_page = [&](int buf, int pg) {
-        const char* kt = smem + buf * KBYTES;
-        const char* vt = smem + 2 * KBYTES + buf * VBYTES;
+    auto compute_page = [&](const char* kt, const char* vt, int pg) {
         floatx4_t s[RT][4];
         __builtin_amdgcn_s_setprio(1);
 #pragma unroll
@@ -596,19 +601,25 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 
     // Step pg multiplies page pg while the copies of page pg + 1 are on their way into the
     // other pair of buffers, which the step before has read last.
-    copy_keys(page_lo);
-    copy_values(page_lo);
-    copies_landed(page_lo);
+    copy_keys(page_lo, kb0);
+    copy_values(page_lo, vb0);
+    copies_landed(page_lo, vb0);
     __syncthreads();
-    for (int pg = page_lo; pg <= page_hi; ++pg) {
-        if (pg < page_hi) {
-            copy_keys(pg + 1);
-            copy_values(pg + 1);
-        }
-        if (wave_has_rows && pg * 64 <= pmax && pg * 64 + 63 >= w_lo) compute_page(pg & 1, pg);
-        copies_landed(pg + 1);
-        __syncthreads();
+#define TL_PAGE(PG, KCUR, VCUR, KNEXT, VNEXT)                                                    \
+    {                                                                                            \
+        if ((PG) < page_hi) {                                                                    \
+            copy_keys((PG) + 1, KNEXT);                                                          \
+            copy_values((PG) + 1, VNEXT);                                                        \
+        }                                                                                        \
+        if (wave_has_rows && (PG) * 64 <= pmax && (PG) * 64 + 63 >= w_lo) compute_page(KCUR, VCUR, PG); \
+        copies_landed((PG) + 1, VNEXT);                                                          \
+        __syncthreads();                                                                         \
     }
+    for (int pg = page_lo; pg <= page_hi; pg += 2) {       // the first page in kb0, vb0, then in turn
+        TL_PAGE(pg, kb0, vb0, kb1, vb1)
+        if (pg + 1 <= page_hi) TL_PAGE(pg + 1, kb1, vb1, kb0, vb0)
+    }
+#undef TL_PAGE
 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -637,14 +648,7 @@ static void launch_attention_tiled_rt(dim3 grid, int slots, hipStream_t stream, 
     constexpr int HDM = DS * 32;
     const int total = (int)(grid.x * grid.y);
     const int pair_from = (grid.z == 1 && total > 1 && total <= slots && total % 2 == 0) ? total / 2 : 0;
-    const size_t shmem = 2 * (size_t)(64 * HDM * 2 + HDM * 64 * 2);
-    static bool raised = false;
-    if (!raised) {
-        hipFuncSetAttribute((const void*)attention_tiled_kernel<DS, FULL, RT>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        raised = true;
-    }
-    attention_tiled_kernel<DS, FULL, RT><<<grid, 256, shmem, stream>>>(
+    attention_tiled_kernel<DS, FULL, RT><<<grid, 256, 0, stream>>>(
         q, k, v, q_start, start_pos, table, table_stride, out, H, Hkv, hd, sl2, window, pair_from);
 }
 

@@ -72,6 +72,38 @@ def _tiled_for(rows: int, w: torch.Tensor, gate: bool = False):
     return T.tiled_of(w, gate)
 
 
+def _library_slices(M: int, N: int, K_: int, device) -> int:
+    """Slices of the inner size for a product of more than 64 rows through the vendor library.
+    Its kernels give every 128 x 128 tile (or so) of the result to one workgroup that walks the
+    whole inner size: a few hundred rows make fewer tiles than the chip has compute units, and
+    a long inner size makes each of them slow (512 rows times the feed-forward's second matrix
+    of the 8B shape: 128 tiles, 88 us = 0.68 PFLOP/s).  Cut into S slices, run as one batched
+    product with float32 results, the tiles are S times as many (60 us with four slices); the
+    kernels that add the slices are the ones that follow the product anyway (residual sum and
+    norm, rotation and cache write).  Measured on 256 compute units at 128..2048 rows: the
+    slices pay while they bring the tiles up to about 2.5 per compute unit, more for a longer
+    inner size (the float32 partial sums, S * M * N * 4 bytes written and read, are then the
+    smaller part), and never for the gate product, whose result is seven times its x."""
+    if K_ % 8 or M <= 0:
+        return 1
+    tiles = ((M + 127) // 128) * ((N + 127) // 128)
+    want = 2.5 * _compute_units(device) * (K_ / 4096.0) ** 0.5 / tiles
+    S = 1
+    while 2 * S <= want and 2 * S <= 8 and K_ % (16 * S) == 0 and K_ // (2 * S) >= 1024:
+        S *= 2
+    return S
+
+
+def _library_partial_sums(x: torch.Tensor, w: torch.Tensor, S: int) -> torch.Tensor:
+    """float32 [S, M, N]: x W^T over each of S equal slices of the inner size, as one batched
+    product of the vendor library over views of x and w (nothing is copied)."""
+    M, K_ = x.shape
+    N = w.shape[0]
+    xs = x.view(M, S, K_ // S).permute(1, 0, 2)
+    ws = w.view(N, S, K_ // S).permute(1, 2, 0)
+    return torch.bmm(xs, ws, out_dtype=torch.float32)
+
+
 class HalfNormed:
     """Rows of an RMS norm in two halves, as the few-row product that completed the residual
     stream left them: ``xg`` = bfloat16(residual * norm weight) (``gemm_bf16.ChunkedRows``
@@ -138,6 +170,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return rows if may_stay_sliced else rows.rows()
     if out_dtype == torch.float32:
         return _fast().wide_f32_out(x, w)
+    if M > _wide().MAX_ROWS and w.shape[0] % 4 == 0 and x.is_contiguous() and w.is_contiguous():
+        S = _library_slices(M, w.shape[0], x.shape[1], x.device)
+        if S > 1:
+            rows = SlicedRows(_library_partial_sums(x, w, S), out_dtype)
+            return rows if may_stay_sliced else rows.rows()
     return torch.matmul(x, w.t())
 
 
@@ -162,6 +199,11 @@ def linear_into(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, then_n
             return _wide().sum_add_norm(residual, T.partial_sums(x, t), weight, eps)
         if _sliced_is_faster(x.shape[0], w.shape[0], x.shape[1]):
             return _wide().product_into(x, w, residual, weight, eps)
+        if x.shape[0] > _wide().MAX_ROWS and w.shape[0] % 4 == 0 and w.shape[0] <= 16384 \
+                and x.is_contiguous() and w.is_contiguous():
+            S = _library_slices(x.shape[0], w.shape[0], x.shape[1], x.device)
+            if S > 1:
+                return _wide().sum_add_norm(residual, _library_partial_sums(x, w, S), weight, eps)
         if form is not None:
             return K.add_rmsnorm(residual, torch.matmul(x, w.t()), weight, eps)
     _linear_into(x, w, residual)

@@ -189,6 +189,44 @@ def test_products_over_weights_in_operand_order(M, N, K_):
         close(T.product_gated(x.to(DEV), tg), a * torch.sigmoid(a) * b, 1.5e-2)
 
 
+@pytest.mark.parametrize("M,N,K_", [(300, 512, 4096), (129, 256, 8192), (700, 1024, 2048)])
+def test_many_row_products_in_slices_of_the_inner_size(M, N, K_):
+    """More than 64 rows times a matrix with few tiles: the vendor library's batched product
+    over slices of the inner size (float32 partial sums), added by the kernel that completes
+    the residual stream and norms it, or kept for a reader that adds them; against float64."""
+    from gpt_fast_amd.ops import linear as L
+    torch.manual_seed(M)
+    S = L._library_slices(M, N, K_, torch.device(DEV))
+    assert S > 1 and K_ % S == 0
+    x = bf(torch.randn(M, K_, device=DEV))
+    w = bf(torch.randn(N, K_, device=DEV) / math.sqrt(K_))
+    ref = x.double() @ w.double().T
+    part = L._library_partial_sums(x, w, S)
+    assert part.shape == (S, M, N) and part.dtype == torch.float32 and part.is_contiguous()
+    per = K_ // S
+    for i in (0, S - 1):
+        close(part[i], x[:, i * per:(i + 1) * per].double() @ w[:, i * per:(i + 1) * per].double().T, 2e-5)
+    res0 = torch.randn(M, N, device=DEV)
+    g, eps = (1 + 0.1 * torch.randn(N, device=DEV)).float(), 1e-5
+
+    class Norm:
+        def row_and_column_form(self):
+            return g, eps
+
+    res = res0.clone()
+    xn = L.linear_into(x, w, res, Norm())
+    r = res0.double() + ref
+    close(res, r, 2e-5)
+    close(xn, r * torch.rsqrt((r ** 2).mean(-1, keepdim=True) + eps) * g.double(), 6e-3)
+    res = res0.clone()
+    assert L.linear_into(x, w, res) is None
+    close(res, r, 2e-5)
+    rows = L.linear(x, w, may_stay_sliced=True)
+    assert isinstance(rows, L.SlicedRows) and rows.part.shape[0] == S
+    close(rows.rows(), ref, 1e-2)
+    close(L.linear(x, w), ref, 1e-2)
+
+
 def test_sliced_product_equals_its_slices_added_in_order():
     from gpt_fast_amd.ops import gemm_wide_bf16 as W
     torch.manual_seed(15)

@@ -22,6 +22,7 @@
 // waves; each writes an unnormalised partial result with its maximum and sum, and a
 // second kernel combines them in split order.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
@@ -362,10 +363,11 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
 // registers in between) while earlier pages are multiplied.
 //
 // The arithmetic is that of the kernel above, a page (64 keys) at a time.
-// RT row tiles of 16 per wave: 2 (128 rows per workgroup) where the grid exceeds what the chip
-// holds at once and throughput counts (an operand read from LDS then serves two matrix
-// instructions); 1 (64 rows) for grids that are resident at once, where the time is that of
-// the workgroup with the most keys and twice as many, lighter workgroups shorten it.
+// RT row tiles of 16 per wave: 2 (128 rows per workgroup) once such workgroups fill the slots
+// of the chip (two per compute unit): an operand read from LDS then serves two matrix
+// instructions; 1 (64 rows) for smaller grids, which need the workgroups more than the reuse
+// (measured at head size 128, 8 kv heads: 1,536 tokens 37.8 us against 43.6, 2,048 tokens
+// 58.7 against 54.7).
 #define TL_WAVES 4
 
 // FULL: the head size is exactly the one the tiles are laid out for (no edge tests).
@@ -516,110 +518,184 @@ __global__ __launch_bounds__(256, 2) void attention_tiled_kernel(
 #pragma unroll
     for (int ds = 0; ds < DS; ++ds) k_off[ds] = (ds * 4 + lg) * 512 + li * 16;
 
-    // One page (64 keys) at a time: all scores first, then the softmax of the row tiles, then
-    // the second product.  The wave's priority is raised while it issues matrix instructions,
-    // so that the other waves of the SIMD fill the gaps with their vector work and not the
-    // other way round.
-    auto compute_page = [&](const char* kt, const char* vt, int pg) {
-        floatx4_t s[RT][4];
-        __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-        for (int kt16 = 0; kt16 < 4; ++kt16) {
-            Frag kf[DS];
+    // The pages this wave has keys in (none: hi < lo).
+    const int w_page_lo = (w_lo >> 6) > page_lo ? (w_lo >> 6) : page_lo;
+    const int w_page_hi = wave_has_rows ? pmax >> 6 : -1;
+
+    // A step works on two pages at once, so that matrix and vector instructions of one wave
+    // have nothing to wait for in each other: the scores of page p + 1 (keys times queries) are
+    // multiplied while the exponentials of page p are taken, and the second product of page p
+    // (values times probabilities) while the row maxima of page p + 1 are.  The source gives
+    // the order - one or two matrix instructions, then a few vector instructions that do not
+    // need their result - and scheduling fences keep it.  `sc` holds the scores of page p,
+    // masked, from the step before; m already covers them.
+    floatx4_t sc[RT][4];
+    auto step = [&](auto cur_tag, auto nxt_tag, int pg, const char* kt, const char* vt) {
+        constexpr bool CUR = decltype(cur_tag)::value, NXT = decltype(nxt_tag)::value;
+        floatx4_t s2[RT][4];
+        Frag pf[RT][2];
+        Frag kf[4][DS];
+        Frag vf[DT][2];
+        float neg_m[RT], sum[RT], p_e[RT][4];
+        constexpr int KAHEAD = RT == 1 ? 4 : 2;            // key blocks requested ahead of their use
+        constexpr int VAHEAD = RT == 1 ? DT : (DT + 1) / 2;
+        auto read_keys = [&](int kt16) {
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds)
-                kf[ds].u = (FULL || ds * 32 + lg * 8 < hd)
-                               ? *(const uint4*)(kt + (kt16 >> 1) * 64 * hdr + (kt16 & 1) * 256 + k_off[ds])
-                               : make_uint4(0, 0, 0, 0);
+                kf[kt16][ds].u = (FULL || ds * 32 + lg * 8 < hd)
+                                     ? *(const uint4*)(kt + (kt16 >> 1) * 64 * hdr + (kt16 & 1) * 256 + k_off[ds])
+                                     : make_uint4(0, 0, 0, 0);
+        };
+        auto read_values = [&](int dt) {
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) vf[dt][hb].u = *(const uint4*)(vt + (dt * 2 + hb) * 1024 + lane * 16);
+        };
+        if (NXT) {
+#pragma unroll
+            for (int kt16 = 0; kt16 < KAHEAD; ++kt16) read_keys(kt16);
+        }
+        if (CUR) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                s[rt][kt16] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ds = 0; ds < DS; ++ds)
-                    s[rt][kt16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ds].v, qf[rt][ds].v, s[rt][kt16], 0, 0, 0);
+                neg_m[rt] = (m[rt] == -INFINITY) ? 0.f : -m[rt];
+                sum[rt] = 0.f;
             }
         }
-        __builtin_amdgcn_s_setprio(0);
-        const bool masked = pg * 64 + 63 > pmin || (window > 0 && pg * 64 < pmax - window + 1);
-        const int key0 = pg * 64 + lg * 8;                 // this lane's keys: key0 .. +7, key0 + 32 .. +39
-        Frag pf[RT][2];
+        __builtin_amdgcn_sched_barrier(0);
+        // scores of page pg + 1 | exponentials of page pg
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            float sv[16];                                  // raw scores; -inf where masked
-            if (masked) {
-                const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
+        for (int kt16 = 0; kt16 < 4; ++kt16) {
+            if (NXT && kt16 + KAHEAD < 4) read_keys(kt16 + KAHEAD);
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int key = key0 + (e >> 3) * 32 + (e & 7);
-                    sv[e] = (key <= rpos[rt] && key >= first) ? s[rt][e >> 2][e & 3] : -INFINITY;
+            for (int ds = 0; ds < DS; ++ds) {
+                if (NXT) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        s2[rt][kt16] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            kf[kt16][ds].v, qf[rt][ds].v, ds == 0 ? floatx4_t{0.f, 0.f, 0.f, 0.f} : s2[rt][kt16], 0, 0, 0);
                 }
-            } else {
+                if (CUR) {
+                    // the four scores of key block kt16, one per matrix instruction (a head
+                    // size of 64 has two per block: two scores each)
+                    constexpr int PER = 4 / DS;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) sv[e] = s[rt][e >> 2][e & 3];
-            }
-            float mx = fmaxf(fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                                   fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7]))),
-                             fmaxf(fmaxf(fmaxf(sv[8], sv[9]), fmaxf(sv[10], sv[11])),
-                                   fmaxf(fmaxf(sv[12], sv[13]), fmaxf(sv[14], sv[15]))));
-            mx = max_over_lane_groups(mx) * scale_log2;    // scale > 0: the order is kept
-            if (__builtin_amdgcn_ballot_w64(mx > m[rt] + TL_SLACK) != 0) {
-                // some row's maximum moved far: raise every row's reference and rescale
-                const float m_new = fmaxf(m[rt], mx);
-                const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[rt] - m_new);
-                l[rt] *= alpha;
-                m[rt] = m_new;
+                    for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= alpha;
-            }
-            const float neg_m = (m[rt] == -INFINITY) ? 0.f : -m[rt];
-            float sum = 0.f;
+                        for (int j = ds * PER; j < (ds + 1) * PER; ++j) {
+                            p_e[rt][j] = __builtin_amdgcn_exp2f(fmaf(sc[rt][kt16][j], scale_log2, neg_m[rt]));
+                            sum[rt] += p_e[rt][j];
+                            // computed here, between the matrix instructions, not where the
+                            // second product uses it (the compiler would sink it there)
+                            asm volatile("" : "+v"(p_e[rt][j]), "+v"(sum[rt]));
+                        }
+                        if (ds == DS - 1) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float p = __builtin_amdgcn_exp2f(fmaf(sv[e], scale_log2, neg_m));
-                sum += p;
-                pf[rt][e >> 3].e[e & 7] = float_to_bf16(p);
+                            for (int j = 0; j < 4; ++j)
+                                pf[rt][kt16 >> 1].e[(kt16 & 1) * 4 + j] = float_to_bf16(p_e[rt][j]);
+                            if (kt16 & 1) asm volatile("" : "+v"(pf[rt][kt16 >> 1].u.z), "+v"(pf[rt][kt16 >> 1].u.w));
+                            else asm volatile("" : "+v"(pf[rt][kt16 >> 1].u.x), "+v"(pf[rt][kt16 >> 1].u.y));
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            l[rt] += sum;
         }
-        __builtin_amdgcn_s_setprio(1);
+        if (CUR) {
 #pragma unroll
-        // every tile of dims is multiplied, also those beyond a smaller head (what LDS holds
-        // there goes into accumulators that are never stored): no branch directly behind a
-        // matrix instruction (see the wave-level kernel above)
+            for (int rt = 0; rt < RT; ++rt) l[rt] += sum[rt];
+#pragma unroll
+            for (int dt = 0; dt < VAHEAD; ++dt) read_values(dt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float mx[RT];
+        if (NXT) {
+            const int p2 = pg + 1;
+            const bool masked = p2 * 64 + 63 > pmin || (window > 0 && p2 * 64 < pmax - window + 1);
+            if (masked) {
+                const int key0 = p2 * 64 + lg * 8;         // this lane's keys: key0 .. +7, key0 + 32 .. +39
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    const int first = (window > 0) ? rpos[rt] - window + 1 : 0;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = key0 + (e >> 3) * 32 + (e & 7);
+                        if (!(key <= rpos[rt] && key >= first)) s2[rt][e >> 2][e & 3] = -INFINITY;
+                    }
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) mx[rt] = -INFINITY;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // second product of page pg | row maxima of page pg + 1
+#pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
+            if (CUR) {
+                if (dt + VAHEAD < DT) read_values(dt + VAHEAD);
+                // every tile of dims is multiplied, also those beyond a smaller head (what LDS
+                // holds there goes into accumulators that are never stored)
 #pragma unroll
-            for (int hb = 0; hb < 2; ++hb) {
-                Frag vf;
-                vf.u = *(const uint4*)(vt + (dt * 2 + hb) * 1024 + lane * 16);
+                for (int hb = 0; hb < 2; ++hb) {
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
+                    for (int rt = 0; rt < RT; ++rt)
+                        o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][hb].v, pf[rt][hb].v, o[rt][dt], 0, 0, 0);
+                }
+            }
+            if (NXT) {
+                // DT is 4 or 8: the sixteen scores of a row tile in DT steps
+                constexpr int PER = 16 / DT;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                    for (int e = dt * PER; e < (dt + 1) * PER; ++e) mx[rt] = fmaxf(mx[rt], s2[rt][e >> 2][e & 3]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (NXT) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const float top = max_over_lane_groups(mx[rt]) * scale_log2;   // scale > 0: the order is kept
+                if (__builtin_amdgcn_ballot_w64(top > m[rt] + TL_SLACK) != 0) {
+                    // some row's maximum moved far: raise every row's reference and rescale
+                    const float m_new = fmaxf(m[rt], top);
+                    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[rt] - m_new);
+                    l[rt] *= alpha;
+                    m[rt] = m_new;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= alpha;
+                }
+#pragma unroll
+                for (int kt16 = 0; kt16 < 4; ++kt16) sc[rt][kt16] = s2[rt][kt16];
             }
         }
-        __builtin_amdgcn_s_setprio(0);
     };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
 
-    // Step pg multiplies page pg while the copies of page pg + 1 are on their way into the
-    // other pair of buffers, which the step before has read last.
+    // Step pg reads the keys of page pg + 1 and the values of page pg, while the copies of the
+    // keys of page pg + 2 and the values of page pg + 1 are on their way into the buffers that
+    // the step before has read last.  The first step (pg = page_lo - 1) has no page of its own.
     copy_keys(page_lo, kb0);
-    copy_values(page_lo, vb0);
-    copies_landed(page_lo, vb0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-#define TL_PAGE(PG, KCUR, VCUR, KNEXT, VNEXT)                                                    \
+#define TL_STEP(PG, KNEXT, KFREE, VCUR, VFREE)                                                   \
     {                                                                                            \
-        if ((PG) < page_hi) {                                                                    \
-            copy_keys((PG) + 1, KNEXT);                                                          \
-            copy_values((PG) + 1, VNEXT);                                                        \
-        }                                                                                        \
-        if (wave_has_rows && (PG) * 64 <= pmax && (PG) * 64 + 63 >= w_lo) compute_page(KCUR, VCUR, PG); \
-        copies_landed((PG) + 1, VNEXT);                                                          \
+        if ((PG) + 2 <= page_hi) copy_keys((PG) + 2, KFREE);                                     \
+        if ((PG) + 1 <= page_hi) copy_values((PG) + 1, VFREE);                                   \
+        const bool cur = (PG) >= w_page_lo && (PG) <= w_page_hi;                                 \
+        const bool nxt = (PG) + 1 >= w_page_lo && (PG) + 1 <= w_page_hi;                         \
+        if (cur && nxt) step(Yes{}, Yes{}, PG, KNEXT, VCUR);                                     \
+        else if (cur) step(Yes{}, No{}, PG, KNEXT, VCUR);                                        \
+        else if (nxt) step(No{}, Yes{}, PG, KNEXT, VCUR);                                        \
+        copies_landed((PG) + 1, VFREE);                                                          \
         __syncthreads();                                                                         \
     }
-    for (int pg = page_lo; pg <= page_hi; pg += 2) {       // the first page in kb0, vb0, then in turn
-        TL_PAGE(pg, kb0, vb0, kb1, vb1)
-        if (pg + 1 <= page_hi) TL_PAGE(pg + 1, kb1, vb1, kb0, vb0)
+    for (int pg = page_lo - 1; pg <= page_hi; pg += 2) {
+        TL_STEP(pg, kb0, kb1, vb1, vb0)
+        if (pg + 1 <= page_hi) TL_STEP(pg + 1, kb1, kb0, vb0, vb1)
     }
-#undef TL_PAGE
+#undef TL_STEP
 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -665,8 +741,8 @@ static void launch_attention_tiled(int max_rows, int n_seqs, int row_tiles, hipS
         slots = 2 * (cus > 0 ? cus : 1);
     }
     const int tiles128 = (max_rows + 127) / 128;
-    if (row_tiles == 0) row_tiles = ((long)tiles128 * Hkv * n_seqs <= slots) ? 1 : 2;
-    if (row_tiles == 1)                                    // resident at once: lighter workgroups
+    if (row_tiles == 0) row_tiles = ((long)tiles128 * Hkv * n_seqs < slots) ? 1 : 2;
+    if (row_tiles == 1)
         launch_attention_tiled_rt<DS, FULL, 1>(dim3((max_rows + 63) / 64, Hkv, n_seqs), slots, stream, q, k, v,
                                                q_start, start_pos, table, table_stride, out, H, Hkv, hd, sl2, window);
     else

@@ -12,14 +12,25 @@ MAX_SPLITS = 32
 # Single-token steps.  A wave takes its keys one 32-key block after another (0.6 us each, two
 # in flight); splitting a context over several workgroups shortens that chain but costs a
 # second kernel that sums the splits (3 to 4 us with its boundary).  Measured on contexts of
-# 128 to 16,384 keys and 1 to 64 sequences (8 kv heads, head size 128): no split pays while a
-# wave has at most SPLIT_FROM_BLOCKS blocks; 128 workgroups already stream the cache at the
-# memory's rate, so splits only make up for missing workgroups, never beyond FILL_GROUPS; a
-# split is left with two blocks per wave at least.
+# 128 to 16,384 keys and 1 to 64 sequences (8 kv heads, head size 128, 256 compute units): no
+# split pays while a wave has at most SPLIT_FROM_BLOCKS blocks; a workgroup on every second
+# compute unit already streams the cache at the memory's rate, so splits only make up for
+# missing workgroups, never beyond one per compute unit; a split is left with two blocks per
+# wave at least.
 SPLIT_FROM_BLOCKS = 6
-FILL_GROUPS = 256
-STREAMING_GROUPS = 128
-LONG_BLOCKS = 48           # with 128..255 workgroups, two splits from this many blocks per wave on
+LONG_BLOCKS = 48           # with a workgroup on every second compute unit or more, two splits
+                           # from this many blocks per wave on
+
+_units = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device (asked once each)."""
+    index = torch.cuda.current_device() if device is None else torch.device(device).index
+    n = _units.get(index)
+    if n is None:
+        n = _units[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return n
 
 
 TILED_MIN_ROWS = 64        # prompts with at least this many (token, head) rows per kv head use
@@ -28,22 +39,25 @@ PREFILL_ROW_TILES = 4      # 16-row tiles per wave for prompts
 TILED_ROW_TILES = 0        # of the workgroup-tiled kernel: 1 or 2, or 0 = by the size of the grid
 
 
-def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int):
+def plan(n_seqs: int, max_q_len: int, H: int, G: int, hd: int, table_width: int, units=None):
     """(row tiles per wave, waves per workgroup, workgroups per sequence and kv head,
-    context splits) for a step."""
+    context splits) for a step on a device of ``units`` compute units (default: the current
+    device's)."""
     R = H // G
     if max_q_len == 1:
+        fill = units or compute_units()
+        streaming = (fill + 1) // 2
         rt = 1
         nw = 4 if hd <= 128 else 2
         tiles = (R + 15) // 16
         groups = n_seqs * G * tiles                      # workgroups without any split
         blocks = (table_width * 2 + nw - 1) // nw          # key blocks per wave at most
-        if blocks <= SPLIT_FROM_BLOCKS or groups >= FILL_GROUPS:
+        if blocks <= SPLIT_FROM_BLOCKS or groups >= fill:
             splits = 1
-        elif groups >= STREAMING_GROUPS:
+        elif groups >= streaming:
             splits = 2 if blocks >= LONG_BLOCKS else 1
         else:
-            splits = min((blocks + 1) // 2, (FILL_GROUPS + groups - 1) // groups, MAX_SPLITS)
+            splits = min((blocks + 1) // 2, (fill + groups - 1) // groups, MAX_SPLITS)
         return rt, nw, tiles, splits
     rt = PREFILL_ROW_TILES if hd <= 128 else min(PREFILL_ROW_TILES, 2)
     rows = max_q_len * R

@@ -4,11 +4,16 @@ reference's linears (model.py:110, 174-175, 222-224), with the epilogues the blo
 float32 engine: the library's own float32 kernel, for every shape (a true 32-bit
 product; one fused-multiply-add chain per output).
 
-bfloat16 engine: hand-written kernels for the few-row products of decoding (up to 16
-rows; weights are streamed once; see csrc/gemm_bf16.hip); the vendor matrix library,
-through ``torch.matmul``, for products of more rows - the reference uses the vendor
-library for these as well - except where a hand-written kernel for 17..64 rows
-(csrc/gemm_wide_bf16.hip) measures faster.  Accumulation is float32 everywhere.
+bfloat16 engine, by the rows of x: up to 16, hand-written kernels that stream the weights
+once (csrc/gemm_bf16.hip; up to 24 rows inside a layer's chain where a matrix has no
+tiled copy); 17..64, hand-written kernels over a second copy of the weights in the matrix
+cores' operand order (csrc/gemm_tiled_bf16.hip), and without that copy the sliced kernel of
+csrc/gemm_wide_bf16.hip or the vendor library, whichever measures faster for the shape;
+more rows, the vendor matrix library through ``torch.matmul`` - the reference uses the
+vendor library for these as well - cut into slices of the inner size (``torch.bmm``) where
+the result has too few tiles to fill the chip.  A sliced product leaves float32 partial
+sums that the kernel behind it adds in slice order (:class:`SlicedRows`).  Accumulation is
+float32 everywhere.
 """
 from typing import Optional
 

@@ -504,3 +504,29 @@ def test_a_part_can_ask_for_a_field_of_its_own_in_the_steps_description():
     assert off % 4 == 0 and lay.key() != BatchLayout(4, 2, 2, {0: 2}).key()
     with pytest.raises(ValueError, match="tokens"):
         BatchLayout(1, 1, 1, {}, extra=[StepField("tokens", lambda n, b: 1, fill)])
+
+
+def test_dispatch_thresholds_follow_the_number_of_compute_units():
+    """Decisions that depend on the chip take its number of compute units as an argument:
+    the context splits of single-token attention (never more workgroups than compute units,
+    none where every second unit has one and the chain is short) and the slices of a
+    many-row library product (as many as bring the result tiles to about 2.5 per unit)."""
+    from gpt_fast_amd.ops import attention_bf16 as A
+    from gpt_fast_amd.ops import linear as L
+    # one sequence, 8 kv heads, 4,096 keys: 8 workgroups without a split, 32 blocks per wave
+    assert A.plan(1, 1, 32, 8, 128, 64, units=256)[3] == 16        # two blocks per wave at least
+    assert A.plan(1, 1, 32, 8, 128, 64, units=64)[3] == 8          # 8 x 8 = 64 workgroups
+    assert A.plan(1, 1, 32, 8, 128, 64, units=8)[3] == 1           # already one per unit
+    assert A.plan(16, 1, 32, 8, 128, 64, units=256)[3] == 1        # 128 workgroups stream
+    assert A.plan(16, 1, 32, 8, 128, 512, units=256)[3] == 2       # ... unless the chain is long
+    assert A.plan(1, 1, 32, 8, 128, 3, units=256)[3] == 1          # a short context: no split
+    L._units["fake256"], L._units["fake64"] = 256, 64
+    try:
+        assert L._library_slices(512, 4096, 14336, "fake256") == 8
+        assert L._library_slices(2048, 4096, 14336, "fake256") == 2
+        assert L._library_slices(2048, 4096, 4096, "fake256") == 1
+        assert L._library_slices(2048, 4096, 14336, "fake64") == 1
+        assert L._library_slices(512, 4096, 4096, "fake256") == 4
+        assert L._library_slices(300, 200, 96, "fake256") == 1     # a short inner size is never cut
+    finally:
+        del L._units["fake256"], L._units["fake64"]

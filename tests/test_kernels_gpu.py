@@ -859,6 +859,21 @@ def test_wide_matrices_at_nine_to_sixteen_rows(M):
     close(kp, kp2, 1e-2)
     assert torch.equal(vp, vp2)
     assert torch.equal(kp == 0, kp2 == 0) and torch.equal(vp == 0, vp2 == 0)
+    # and against float64 of the whole: product, rotation by interleaved pairs, the page and
+    # place each token's keys and values went to
+    rows = (xn.double() @ wq.double().T).view(M, H + 2 * G_, hd).cpu()
+    ang = tok_pos.cpu().float()[:, None] * freqs.cpu()[None, :]
+    c, s_ = torch.cos(ang.double())[:, None, :], torch.sin(ang.double())[:, None, :]
+    ref = rows.clone()
+    a, b = rows[:, :H + G_, 0::2], rows[:, :H + G_, 1::2]
+    ref[:, :H + G_, 0::2] = a * c - b * s_
+    ref[:, :H + G_, 1::2] = b * c + a * s_
+    close(q, ref[:, :H], 1e-2)
+    kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
+    for n in range(M):
+        p_ = int(tok_pos[n])
+        close(kc[4 * n + p_ // 64, :, p_ % 64], ref[n, H:H + G_], 1e-2)
+        close(vc[4 * n + p_ // 64, :, :, p_ % 64], ref[n, H + G_:], 1e-2)
 
 
 @pytest.mark.parametrize("H,G_,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (32, 8, 128, 128), (2, 2, 32, 0)])
@@ -888,6 +903,25 @@ def test_projection_rotation_and_cache_write_in_one_kernel(H, G_, hd, rot):
     close(kp, kp2, 1e-2)
     assert torch.equal(vp, vp2)                        # values are not rotated: same products
     assert torch.equal(kp == 0, kp2 == 0) and torch.equal(vp == 0, vp2 == 0)   # same places written
+    # and a reference of their own, in float64: the product of the normed rows, rotated by
+    # interleaved pairs (model.py:284-292), read back from the pages the table names
+    rows = (xn.double() @ w.double().T).view(M, H + 2 * G_, hd).cpu()
+    ref = rows.clone()
+    if rot:
+        ang = torch.tensor(pos, dtype=torch.float32)[:, None] * freqs.cpu()[None, :]
+        c, s_ = torch.cos(ang.double())[:, None, :], torch.sin(ang.double())[:, None, :]
+        a, b = rows[:, :H + G_, 0:rot:2], rows[:, :H + G_, 1:rot:2]
+        ref[:, :H + G_, 0:rot:2] = a * c - b * s_
+        ref[:, :H + G_, 1:rot:2] = b * c + a * s_
+    close(q, ref[:, :H], 1e-2)
+    kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
+    written = torch.zeros(100, 64, dtype=torch.bool)
+    for n in range(M):
+        page = int(table[seq[n], pos[n] // 64])
+        written[page, pos[n] % 64] = True
+        close(kc[page, :, pos[n] % 64], ref[n, H:H + G_], 1e-2)
+        close(vc[page, :, :, pos[n] % 64], ref[n, H + G_:], 1e-2)
+    assert not kc.permute(0, 2, 1, 3)[~written].any() and not vc.permute(0, 3, 1, 2)[~written].any()
     # no pages: q only
     q3 = G.qkv_rope_store(xn, w, freqs, tok_seq, tok_pos, table, None, None, H, G_, hd, rot)
     assert torch.equal(q3, q)

@@ -7,7 +7,7 @@ from ..config.spec import AttentionSpec
 from ..ops import attention as A
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import POSITIONS, Param, Part, Runtime, check_bound, register_mixer
+from .base import POSITIONS, Param, Part, Runtime, add_late, check_bound, register_mixer
 
 
 class Attention(Part):
@@ -61,11 +61,12 @@ class Attention(Part):
         s = self.spec
         return (s.n_heads + 2 * s.n_kv_heads) * s.head_dim
 
-    prepares_norm = True
+    defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 
-    def forward(self, x, batch, entry, residual, then_norm=None, takes_halves=False):
+    def forward(self, x, batch, entry, residual):
         s = self.spec
+        n_rows = x.shape[0]
         q = None
         fused = getattr(self.position, "project_rotate_store", None)
         if fused is not None and L.can_project_rotate_store(x, self.wqkv, s.head_dim):
@@ -76,13 +77,17 @@ class Attention(Part):
                            may_stay_sliced=getattr(self.position, "takes_sliced", False))
             q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
                                                s.head_dim)                  # model.py:201-207
-        # the output projection may take the heads' results in the order it loads them in
-        rows_for_wo = L.takes_chunked_rows(x.shape[0], q.dtype, self.wo, then_norm, takes_halves)
-        y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
-                        self.scale, self.window, for_product=rows_for_wo)   # model.py:209-211
-        if isinstance(y, torch.Tensor):
-            y = y.view(x.shape[0], s.n_heads * s.head_dim)
-        return L.linear_into(y, self.wo, residual, then_norm, takes_halves)  # model.py:215, 162
+
+        def finish(rows, then_norm, takes_halves):
+            # the output projection may take the heads' results in the order it loads them in
+            rows_for_wo = L.takes_chunked_rows(n_rows, q.dtype, self.wo, then_norm, takes_halves)
+            y = A.attention(q, entry.k_pages, entry.v_pages, batch, batch.table(entry.group_id),
+                            self.scale, self.window, for_product=rows_for_wo)   # model.py:209-211
+            if isinstance(y, torch.Tensor):
+                y = y.view(n_rows, s.n_heads * s.head_dim)
+            return L.linear_into(y, self.wo, rows, then_norm, takes_halves)  # model.py:215, 162
+
+        add_late(residual, finish)
 
 
 register_mixer("attention", Attention)

@@ -24,15 +24,20 @@ never ``host_field`` or a host copy - so that a step recorded once can be replay
 later steps of the same shape.  A part without it (the default) makes generation step the
 model without a recording.
 
-Optional, for speed only: a mixer or feed-forward that sets ``prepares_norm = True`` also
-takes ``then_norm=`` (the norm that reads the residual stream after it) and
-``takes_halves=`` and returns that norm's rows if its last kernel produced them on the way,
-else None; with ``takes_halves`` they may be an ``ops.linear.HalfNormed``, which the products
-of ``ops.linear`` accept in place of x, and a part that passes its x only to those sets
-``takes_prepared = True``.  A norm offers this by ``row_and_column_form() -> (column
-weights, eps)``.  A block with ``prepares_norm`` takes ``x=`` (the rows of its first norm,
-``mixer_norm``, if the caller has them), ``then_norm=`` and ``takes_halves=`` and returns
-likewise.  Parts without the flags are called as above and get plain tensors.
+Optional, for speed only: the kernel that completes the residual stream can apply the norm
+that reads it next on its way, if it knows that norm.  It is known when the stream is read
+next, so a part may put off its last kernels until then: a mixer or feed-forward that sets
+``defers_sum = True`` is given the step's :class:`ResidualStream` as ``residual`` and hands it
+a function ``finish(rows, then_norm, takes_halves) -> normed rows | None`` (:func:`add_late`)
+instead of adding into a tensor; the stream calls it when the next reader asks for
+``stream.normed(norm, reader)`` - or for the plain tensor - and nothing else has touched the
+stream in between.  ``takes_halves`` says that the reader accepts the norm in two halves
+(``ops.linear.HalfNormed``, which the products of ``ops.linear`` take in place of x); a part
+that passes its x only to those sets ``takes_prepared = True`` (or the least number of rows
+from which it wants them).  A norm offers the fused form by ``row_and_column_form() ->
+(column weights, eps)``.  A block that sets ``takes_stream = True`` is given the stream
+instead of the tensor and reads it with ``stream.normed``.  Parts and blocks without these
+flags get plain tensors, as the interfaces above say, and lose nothing but the fusion.
 """
 from dataclasses import dataclass
 from typing import Callable, Dict, Tuple
@@ -76,6 +81,57 @@ class Part:
         """Further int32 fields of a step's description that this part reads
         (``engine.batch.StepField``); none by default."""
         return ()
+
+
+class ResidualStream:
+    """The float32 residual stream of a step, ``[N, D]``, with at most one part's last
+    kernels put off until the stream is read next (see the module's text).  Whoever reads it
+    says how: ``normed(norm, reader)`` for the rows of a norm over it, ``tensor`` for the
+    stream itself; both run what was put off first, so the order of the arithmetic is that
+    of the plain wiring."""
+
+    def __init__(self, rows: torch.Tensor):
+        self._rows = rows
+        self._finish = None
+
+    @property
+    def shape(self):
+        return self._rows.shape
+
+    def defer(self, finish: Callable) -> None:
+        """``finish(rows, then_norm, takes_halves)`` adds a part's result into ``rows`` and
+        returns the rows of ``then_norm`` over the sum if its kernel made them, else None."""
+        self._settle(None, False)
+        self._finish = finish
+
+    def _settle(self, norm, takes_halves: bool):
+        finish, self._finish = self._finish, None
+        return None if finish is None else finish(self._rows, norm, takes_halves)
+
+    @property
+    def tensor(self) -> torch.Tensor:
+        self._settle(None, False)
+        return self._rows
+
+    def normed(self, norm, reader=None, rows=None):
+        """The rows of ``norm`` over the stream (``rows``: only these, by index), for
+        ``reader``: from the kernel that completes the stream where it can make them, else by
+        the norm's own kernel."""
+        least = getattr(reader, "takes_prepared", False)
+        halves = bool(least) and self._rows.shape[0] >= int(least)
+        out = self._settle(norm if rows is None else None, halves)
+        if out is not None and rows is None:
+            return out
+        return norm.forward(self._rows, rows=rows)
+
+
+def add_late(residual, finish: Callable) -> None:
+    """For a part with ``defers_sum``: put ``finish`` off on a :class:`ResidualStream`, or run
+    it now on a plain tensor."""
+    if isinstance(residual, ResidualStream):
+        residual.defer(finish)
+    else:
+        finish(residual, None, False)
 
 
 class _Registry:

@@ -1,6 +1,6 @@
 """How norms, mixer, feed-forward and the residual stream are wired in one layer."""
 from ..config.spec import LayerSpec
-from .base import FEED_FORWARDS, MIXERS, NORMS, Part, Runtime, register_block
+from .base import FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, Runtime, register_block
 
 
 class PreNormBlock(Part):
@@ -47,15 +47,10 @@ class PreNormBlock(Part):
             out += list(getattr(child, "step_fields", lambda: ())())
         return out
 
-    # Norm hand-over, optional for every part: a mixer or feed-forward that sets
-    # ``prepares_norm`` takes ``then_norm=`` (the norm that reads the residual stream after
-    # it) and ``takes_halves=`` (whether that norm's reader accepts an ops.linear.HalfNormed
-    # in place of x; a part says so with ``takes_prepared``: True, or the least number of
-    # rows from which it wants them), and returns that norm's rows if
-    # it produced them on the way, else None.  A block that sets ``prepares_norm`` takes
-    # ``x=`` (the rows of its first norm, if the caller has them), ``then_norm=`` and
-    # ``takes_halves=`` in the same sense, and names its first norm ``mixer_norm``.
-    prepares_norm = True
+    # Reads the stream through ``stream.normed`` so that the kernel which completed it can
+    # hand over the norm's rows (parts.base.ResidualStream); parts that do not put off their
+    # sum get the plain tensor.
+    takes_stream = True
 
     @property
     def replayable(self):
@@ -66,27 +61,17 @@ class PreNormBlock(Part):
         return getattr(self.mixer, "takes_prepared", False)
 
     @staticmethod
-    def _wants_halves(part, n_rows: int) -> bool:
-        least = getattr(part, "takes_prepared", False)
-        return bool(least) and n_rows >= int(least)
+    def _residual_for(part, stream):
+        return stream if getattr(part, "defers_sum", False) else stream.tensor
 
-    def forward(self, residual, batch, entry, x=None, then_norm=None, takes_halves=False):
-        if x is None:
-            x = self.mixer_norm.forward(residual)
-        h = None
-        if getattr(self.mixer, "prepares_norm", False):
-            h = self.mixer.forward(x, batch, entry, residual, then_norm=self.feed_forward_norm,
-                                   takes_halves=self._wants_halves(self.feed_forward,
-                                                                   residual.shape[0]))
-        else:
-            self.mixer.forward(x, batch, entry, residual)
-        if h is None:
-            h = self.feed_forward_norm.forward(residual)
-        if then_norm is not None and getattr(self.feed_forward, "prepares_norm", False):
-            return self.feed_forward.forward(h, batch, residual, then_norm=then_norm,
-                                             takes_halves=takes_halves)
-        self.feed_forward.forward(h, batch, residual)
-        return None
+    def forward(self, residual, batch, entry):
+        stream = residual if isinstance(residual, ResidualStream) else ResidualStream(residual)
+        x = stream.normed(self.mixer_norm, reader=self.mixer)
+        self.mixer.forward(x, batch, entry, self._residual_for(self.mixer, stream))
+        h = stream.normed(self.feed_forward_norm, reader=self.feed_forward)
+        self.feed_forward.forward(h, batch, self._residual_for(self.feed_forward, stream))
+        if stream is not residual:
+            stream.tensor                    # a caller with a plain tensor gets the sums now
 
 
 register_block("pre_norm", PreNormBlock)

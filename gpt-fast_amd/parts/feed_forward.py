@@ -1,7 +1,7 @@
 """Gated feed-forward (reference model.py:219-227)."""
 from ..config.spec import GatedFeedForwardSpec
 from ..ops import linear as L
-from .base import Param, Part, Runtime, check_bound, register_feed_forward
+from .base import Param, Part, Runtime, add_late, check_bound, register_feed_forward
 
 
 class GatedFeedForward(Part):
@@ -24,7 +24,7 @@ class GatedFeedForward(Part):
         self.w13, self.w2 = tensors["w13"], tensors["w2"]
 
     replayable = True
-    prepares_norm = True
+    defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
     # x may be an ops.linear.HalfNormed, from one row on (the least number of rows; with the
     # weights streamed past the caches the matrix-core kernel that takes the halves is as fast
     # at one row as the dot-product kernel that does not, and the norm kernel is saved)
@@ -33,8 +33,11 @@ class GatedFeedForward(Part):
     def step_flops(self, q_lens, starts) -> float:
         return 2.0 * sum(q_lens) * 3 * self.spec.hidden * self.spec.dim
 
-    def forward(self, x, batch, residual, then_norm=None, takes_halves=False):
-        return L.gated_into(x, self.w13, self.w2, residual, then_norm, takes_halves)
+    def forward(self, x, batch, residual):
+        # both products wait until the stream is read next: whether the gate's result stays in
+        # the order the second product loads it in depends on the norm that follows
+        add_late(residual, lambda rows, then_norm, takes_halves: L.gated_into(
+            x, self.w13, self.w2, rows, then_norm, takes_halves))
 
 
 register_feed_forward("gated", GatedFeedForward)

@@ -6,7 +6,7 @@ import torch
 from ..config.spec import ModelPlan
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import BLOCKS, NORMS, POSITIONS, Param, Runtime, check_bound
+from .base import BLOCKS, NORMS, POSITIONS, Param, ResidualStream, Runtime, check_bound
 
 
 class DecoderModel:
@@ -135,31 +135,19 @@ class DecoderModel:
             K.scale_cap(residual, plan.embedding_scale)
         if self.input_position is not None:
             self.input_position.add_to_stream(residual, batch)
-        order = plan.order
-        x = None                       # rows of the next norm, if a block produced them
-        for n, run in enumerate(order):                                   # model.py:142-143
+        stream = ResidualStream(residual)
+        for n, run in enumerate(plan.order):                              # model.py:142-143
             block = self.blocks[run.layer]
-            if not getattr(block, "prepares_norm", False):
-                block.forward(residual, batch, cache.entries[n])
-                x = None
-                continue
-            # the head takes plain rows: with its many columns the halves cost more than the
-            # norm kernel they save
-            takes_halves = False
-            if n + 1 < len(order):
-                nxt = self.blocks[order[n + 1].layer]
-                then_norm = getattr(nxt, "mixer_norm", None)
-                least = getattr(nxt, "takes_prepared", False) if getattr(nxt, "prepares_norm", False) else False
-                takes_halves = bool(least) and residual.shape[0] >= int(least)
-            else:
-                then_norm = self.final_norm if getattr(batch, "every_row_wanted", False) else None
-            x = block.forward(residual, batch, cache.entries[n], x=x, then_norm=then_norm,
-                              takes_halves=takes_halves)
+            block.forward(stream if getattr(block, "takes_stream", False) else stream.tensor,
+                          batch, cache.entries[n])
         if batch.n_want == 0:
+            stream.tensor
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32,
                                device=residual.device)
-        if x is None:
-            x = self.final_norm.forward(residual, rows=batch.want_rows)   # model.py:144
+        # the head takes plain rows (no reader named): with its many columns the halves of a
+        # norm cost more than the norm kernel they save
+        every = getattr(batch, "every_row_wanted", False)
+        x = stream.normed(self.final_norm, rows=None if every else batch.want_rows)   # model.py:144
         logits = L.linear(x, self.head, out_dtype=torch.float32)          # model.py:145
         if plan.logit_scale is not None or plan.logit_softcap is not None:
             K.scale_cap(logits, 1.0 if plan.logit_scale is None else plan.logit_scale,

@@ -372,7 +372,9 @@ def test_attention_plan_for_single_token_steps():
     """How a single-token step is cut over waves: pure arithmetic, no kernel.  More sequences
     mean fewer context splits; a split leaves a wave two 32-key blocks of the table's capacity
     at least, there are never more than 32, and short contexts are not split at all."""
-    from gpt_fast_amd.ops.attention_bf16 import MAX_SPLITS, plan
+    import functools
+    from gpt_fast_amd.ops import attention_bf16 as A
+    MAX_SPLITS, plan = A.MAX_SPLITS, functools.partial(A.plan, units=256)   # the chip it was tuned on
     H, G, hd = 32, 8, 128
     for n_seqs in (1, 3, 8, 16, 64, 300):
         last = MAX_SPLITS
@@ -530,3 +532,49 @@ def test_dispatch_thresholds_follow_the_number_of_compute_units():
         assert L._library_slices(300, 200, 96, "fake256") == 1     # a short inner size is never cut
     finally:
         del L._units["fake256"], L._units["fake64"]
+
+
+def test_residual_stream_runs_what_was_put_off_before_any_read():
+    """The stream holds at most one part's last kernels back; every read - the rows of a norm
+    or the tensor itself - runs them first, telling them the norm that reads (only if all
+    rows are read) and whether its reader takes the norm in halves."""
+    from gpt_fast_amd.parts.base import ResidualStream, add_late
+    log = []
+
+    class Norm:
+        def forward(self, residual, rows=None):
+            log.append(("norm", rows))
+            return residual * 2
+
+    class Reader:
+        takes_prepared = 3          # halves from three rows on
+
+    def finish(tag, give=None):
+        def run(rows, then_norm, takes_halves):
+            log.append((tag, then_norm, takes_halves))
+            rows += 1
+            return give
+        return run
+
+    norm = Norm()
+    s = ResidualStream(torch.zeros(4, 2))
+    s.defer(finish("a"))
+    s.defer(finish("b"))                                  # a second part: the first runs now, plainly
+    assert log == [("a", None, False)]
+    out = s.normed(norm, reader=Reader())
+    assert log[1] == ("b", norm, True) and log[2] == ("norm", None)      # no rows handed over: own kernel
+    assert torch.equal(out, torch.full((4, 2), 4.0))
+    s.defer(finish("c", give="handed over"))
+    assert s.normed(norm, reader=None) == "handed over" and log[-1] == ("c", norm, False)
+    s.defer(finish("d", give="ignored"))
+    s.normed(norm, rows=torch.tensor([1]))                # some rows only: no fused norm is asked for
+    assert log[-2] == ("d", None, False) and log[-1][0] == "norm"
+    s.defer(finish("e"))
+    assert float(s.tensor.sum()) == 5 * 8 and log[-1] == ("e", None, False)
+    two = ResidualStream(torch.zeros(2, 2))
+    two.defer(finish("f"))
+    two.normed(norm, reader=Reader())
+    assert ("f", norm, False) in log                      # two rows: below the reader's least
+    plain = torch.zeros(1, 2)
+    add_late(plain, finish("g"))                          # a plain tensor: at once
+    assert log[-1] == ("g", None, False) and float(plain.sum()) == 2

@@ -614,3 +614,79 @@ def test_plan_level_steps_scale_position_and_cap():
     plan2.input_position = plan2.layers[0].mixer.position
     with pytest.raises(TypeError, match="add_to_stream"):
         DecoderModel(plan2, Runtime(torch.float32, DEV))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_block_arrangement_of_its_own_reads_the_stream_and_keeps_the_fused_norms(dtype, monkeypatch):
+    """A third arrangement, registered here: attention, then two gated feed-forwards, each
+    behind a norm of its own.  Its ``forward`` reads the residual stream with
+    ``stream.normed(norm, reader)`` and knows nothing else of how norms ride on the kernels
+    that complete the stream - and still, in a few-row bfloat16 step, only the first norm of
+    the step and the one before the head run as kernels of their own."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.config.spec import ModelPlan, Run
+    from gpt_fast_amd.ops import kernels as KK
+    from gpt_fast_amd.parts import Runtime, register_block
+    from gpt_fast_amd.parts.base import FEED_FORWARDS, NORMS
+    from gpt_fast_amd.parts.block import PreNormBlock
+    from gpt_fast_amd.parts.model import DecoderModel
+
+    class ThreeBranches(PreNormBlock):
+        takes_stream = True
+
+        def __init__(self, spec, rt):
+            super().__init__(spec, rt)
+            self.norm_b = NORMS.build(spec.feed_forward_norm, rt)
+            self.feed_forward_b = FEED_FORWARDS.build(spec.feed_forward, rt)
+
+        def children(self):
+            return {**super().children(), "ffn_norm_b": self.norm_b, "feed_forward_b": self.feed_forward_b}
+
+        def forward(self, stream, batch, entry):
+            x = stream.normed(self.mixer_norm, reader=self.mixer)
+            self.mixer.forward(x, batch, entry, stream)
+            h = stream.normed(self.feed_forward_norm, reader=self.feed_forward)
+            self.feed_forward.forward(h, batch, stream)
+            g = stream.normed(self.norm_b, reader=self.feed_forward_b)
+            self.feed_forward_b.forward(g, batch, stream)
+
+    register_block("toy_three_branches", ThreeBranches)
+
+    arch = gfa.architecture("llama")
+    cfg = arch.read_config(util.TINY_A)
+    base = arch.plan(cfg)
+    layers = [dataclasses.replace(layer, arrangement="toy_three_branches") for layer in base.layers[:2]]
+    plan = ModelPlan(dim=cfg.hidden_size, vocab_size=cfg.vocab_size, layers=layers,
+                     order=[Run(0), Run(1)], final_norm=base.final_norm)
+    compute = torch.float32 if dtype == "float32" else torch.bfloat16
+    model = DecoderModel(plan, Runtime(compute, DEV))
+    w = _random_parameters(model, 33)
+    roles = {name: p.role for name, p in model.parameters().items()}
+    w = {k: (v.to(compute).float() if roles[k] == "matrix" else v) for k, v in w.items()}   # as the engine holds them
+    eng = gfa.Engine.from_plan(plan, {k: (v.to(compute) if roles[k] == "matrix" else v).to(DEV)
+                                      for k, v in w.items()}, dtype, DEV, max_tokens=1024)
+    pcfg = plain.config_from_dict(util.TINY_A)
+    toks = util.random_tokens(cfg.vocab_size, 70, 9)
+
+    x = w["tok_embeddings.weight"][torch.tensor(toks)]
+    for n in range(2):
+        p = f"layers.{n}."
+        x = _plain_attention_block(x, w, p, pcfg)
+        x = _plain_dense_ffn(x, w, p, pcfg)
+        xn = plain.rms_norm(x, w[p + "ffn_norm_b.weight"], pcfg["eps"])
+        w13 = w[p + "feed_forward_b.w13"]
+        x = x + plain.feed_forward(xn, w13[:w13.shape[0] // 2], w13[w13.shape[0] // 2:], w[p + "feed_forward_b.w2"])
+    want = plain.rms_norm(x, w["norm.weight"], pcfg["eps"]) @ w["output.weight"].T
+    _steps_equal_whole(eng, toks, want, cfg.vocab_size, TOL_F32 if dtype == "float32" else util.TOL_BF16)
+
+    if dtype == "bfloat16":
+        from gpt_fast_amd import Entry
+        calls = []
+        real = KK.rmsnorm
+        monkeypatch.setattr(KK, "rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+        slot = eng.start_sequence()
+        eng.step([Entry(slot, toks[:40])])
+        calls.clear()
+        eng.step([Entry(slot, [toks[40]], want=[0])])
+        eng.end_sequence(slot)
+        assert len(calls) == 2, len(calls)     # of seven norms: the step's first and the head's

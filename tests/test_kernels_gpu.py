@@ -227,6 +227,39 @@ def test_many_row_products_in_slices_of_the_inner_size(M, N, K_):
     close(L.linear(x, w), ref, 1e-2)
 
 
+def test_products_of_17_to_64_rows_without_room_for_the_second_copy(monkeypatch):
+    """The tiled copy of a weight matrix is only made while enough of the device's memory
+    stays free; a matrix that was refused one is asked for no other, and its products run on
+    the kernels over the row-major matrix with the same results."""
+    from gpt_fast_amd.ops import gemm_tiled_bf16 as T
+    from gpt_fast_amd.ops import linear as L
+    torch.manual_seed(3)
+    M, N, K_ = 40, 512, 1024
+    x = bf(torch.randn(M, K_, device=DEV))
+    w = bf(torch.randn(N, K_, device=DEV) / math.sqrt(K_))
+    w13 = bf(torch.randn(2 * N, K_, device=DEV) / math.sqrt(K_))
+    ref = x.double() @ w.double().T
+    a = x.double() @ w13.double().T
+    gated = a[:, :N] * torch.sigmoid(a[:, :N]) * a[:, N:]
+    res0 = torch.randn(M, N, device=DEV)
+    with monkeypatch.context() as m:
+        m.setattr(T, "KEEP_FREE_FRACTION", 2.0)            # never enough room
+        assert T.tiled_of(w) is None and w._gfa_tiled_refused
+        assert T.tiled_of(w13, gate=True) is None
+        close(L.linear(x, w), ref, 1e-2)
+        close(L.gated_linear(x, w13), gated, 1.5e-2)
+        res = res0.clone()
+        L.linear_into(x, w, res)
+        close(res, res0.double() + ref, 2e-5 if L._sliced_is_faster(M, N, K_) else 1e-2)
+    assert T.tiled_of(w) is None                           # asked once: the refusal stands
+    w_again = w.clone()
+    assert T.tiled_of(w_again) is not None                 # room now: another tensor gets its copy
+    close(L.linear(x, w_again), ref, 1e-2)
+    res = res0.clone()
+    L.linear_into(x, w_again, res)
+    close(res, res0.double() + ref, 2e-5)
+
+
 def test_sliced_product_equals_its_slices_added_in_order():
     from gpt_fast_amd.ops import gemm_wide_bf16 as W
     torch.manual_seed(15)

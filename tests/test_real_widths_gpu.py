@@ -166,3 +166,28 @@ def test_generation_with_the_recorded_step(wide):
                 assert float(row[tok]) >= bound - slack, (temperature, len(p), i, tok)
     eng.cache.check()
     assert eng.cache.slots.held == 0
+
+
+def test_generation_of_more_sequences_than_the_few_row_kernels_take(wide):
+    """80 sequences at once: the one-token step has 80 rows, more than any hand-written
+    product takes, so its products are the vendor library's - cut into slices of the inner
+    size where the result has few tiles - recorded and replayed like the others."""
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.engine.generate import generate
+    from gpt_fast_amd.ops import linear as L
+    assert L._library_slices(80, wide.cfg["dim"], 11008, torch.device("cuda:0")) > 1      # a feed-forward's second product is cut
+    eng = gfa.Engine.from_folder(wide.folder, dtype="bfloat16", device="cuda:0",
+                                 max_tokens=80 * 64, max_sequences=80)
+    prompts = [util.random_tokens(wide.vocab, 2 + (7 * i) % 23, 300 + i) for i in range(80)]
+    new = 4
+    out = generate(eng, prompts, max_new_tokens=new, temperature=0.0, seed=1, stop_tokens=())
+    again = generate(eng, prompts, max_new_tokens=new, temperature=0.0, seed=1, stop_tokens=(),
+                     use_graph=False)
+    assert again.tokens == out.tokens
+    for b in (0, 33, 79):
+        p, t = prompts[b], out.tokens[b]
+        logits = wide.rows(p + t[:-1], list(range(len(p) - 1, len(p) + new - 1)))
+        for i, tok in enumerate(t):
+            assert float(logits[i][tok]) >= float(logits[i].max()) - TOL_BF16 * float(logits[i].abs().max())
+    eng.cache.check()
+    assert eng.cache.slots.held == 0

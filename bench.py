@@ -13,7 +13,8 @@ the live sequences) per second with the HBM peak; ``points`` holds decode at bat
 Other workloads of the same program: ``--preset`` (another shape), ``--context`` (cache
 positions per sequence), ``--prompt-lens LO:HI`` (prompts of unequal, seeded random lengths;
 adds the ragged prefill's tokens per second), ``--prefill-only`` (just the timed prompt, for
-profiling).  The line also holds what this GPU reaches with a bare read stream and a bare
+profiling), ``--parts`` (no model: a layer's products at ``--batch`` rows and the prompt
+attention at ``--prefill-tokens`` tokens, each timed alone).  The line also holds what this GPU reaches with a bare read stream and a bare
 matrix-instruction loop (``measured_peaks``, and the step's fractions of them beside the
 fractions of the datasheet peaks), the per-step time of each of the ``--runs`` timed regions
 (``ms_per_step`` is their median) and the peak device memory in use.
@@ -119,6 +120,100 @@ def prefill_run(engine, n_tokens, repeats=3):
     return sorted(times)[len(times) // 2]          # median
 
 
+def parts_run(sizes, rows, prompt_tokens):
+    """Microseconds of a layer's products at ``rows`` rows of x, each through the dispatch of
+    ``ops.linear`` as a step calls it (weights cycled through enough copies that none stays in
+    a cache; twenty calls recorded as one HIP graph, so launches do not count), and of the
+    prompt attention over ``prompt_tokens`` tokens of one sequence (least of four rounds)."""
+    import torch
+    from gpt_fast_amd.ops import attention_bf16 as A
+    from gpt_fast_amd.ops import linear as L
+    dev = "cuda:0"
+    D, H, G, hd = sizes["dim"], sizes["n_head"], sizes["n_kv_heads"], sizes["head_dim"]
+    inner, V = sizes["intermediate_size"], sizes["vocab_size"]
+
+    class Norm:
+        def __init__(self, n):
+            self.w = torch.ones(n, device=dev)
+
+        def row_and_column_form(self):
+            return self.w, 1e-5
+
+    def timed(fn, n=20):
+        fn(0)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(n):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            t = a.elapsed_time(b) / n * 1e3
+            best = t if best is None else min(best, t)
+        return best
+
+    products = {}
+    shapes = {"wqkv": ((H + 2 * G) * hd, D), "wo": (D, H * hd), "w13": (2 * inner, D),
+              "w2": (D, inner), "head": (V, D)}
+    for name, (N, K_) in shapes.items():
+        copies = max(2, int(700e6 // (N * K_ * 2)) + 1)
+        ws = [(torch.randn(N, K_, device=dev) * 0.02).bfloat16() for _ in range(copies)]
+        x = torch.randn(rows, K_, device=dev).bfloat16()
+        res = torch.zeros(rows, N, device=dev) if name in ("wo", "w2") else None
+        norm = Norm(N)
+        if name == "wqkv":
+            fn = lambda i: L.linear(x, ws[i % copies], may_stay_sliced=True)    # the rotation adds slices
+        elif name == "w13":
+            fn = lambda i: L.gated_linear(x, ws[i % copies])
+        elif name == "head":
+            fn = lambda i: L.linear(x, ws[i % copies], out_dtype=torch.float32)
+        else:
+            fn = lambda i: L.linear_into(x, ws[i % copies], res, norm)          # sum and next norm ride along
+        for i in range(copies):
+            fn(i)                                  # second copies of the weights are made outside the recording
+        us = timed(fn)
+        products[name] = {"us": round(us, 1), "tb_s": round(N * K_ * 2 / us / 1e6, 2)}
+        log(f"[bench] {name:5s} {rows:3d} rows: {us:7.1f} us  {N * K_ * 2 / us / 1e6:5.2f} TB/s of weights")
+        del ws
+
+    T = prompt_tokens
+    width = (T + 63) // 64
+    k = torch.randn(width + 1, G, 64, hd, device=dev).bfloat16()
+    v = torch.randn(width + 1, G, hd, 64, device=dev).bfloat16()
+    q = torch.randn(T, H, hd, device=dev).bfloat16()
+
+    class Step:
+        n_seqs, max_q_len = 1, T
+        q_start = torch.tensor([0, T], dtype=torch.int32, device=dev)
+        start_pos = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    table = torch.arange(width, dtype=torch.int32, device=dev).view(1, width)
+    best = None
+    for _ in range(4):
+        A.attention(q, k, v, Step, table, hd ** -0.5, 0)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(10):
+            A.attention(q, k, v, Step, table, hd ** -0.5, 0)
+        b.record()
+        torch.cuda.synchronize()
+        t = a.elapsed_time(b) * 100
+        best = t if best is None else min(best, t)
+    flops = 4.0 * H * hd * T * (T + 1) / 2
+    log(f"[bench] prompt attention {T} tokens: {best:.1f} us  {flops / best / 1e6:.0f} TFLOP/s of causal work")
+    return {"products": products,
+            "prompt_attention": {"tokens": T, "us": round(best, 1), "tflops": round(flops / best / 1e6, 1),
+                                 "frac": round(flops / best / 1e6 / MFMA_PEAK_TFLOPS["bf16"], 4)}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,6 +232,9 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="time the prompt and nothing else")
     ap.add_argument("--runs", type=int, default=3,
                     help="timed regions of --steps steps each; the median one is reported")
+    ap.add_argument("--parts", action="store_true",
+                    help="time a layer's products at --batch rows and the prompt attention at "
+                         "--prefill-tokens alone, no model")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1, batch 64 and prefill")
     args = ap.parse_args()
@@ -156,6 +254,10 @@ def main():
     sizes = dict(arch.describe(cfg)) if arch.describe is not None else {}
     n_layers = raw[arch.layer_count_key]
     batch, context = args.batch, args.context
+    if args.parts:
+        print(json.dumps({"metric": f"kernels alone; {args.preset} bf16", "rows": batch,
+                          **parts_run(sizes, batch, args.prefill_tokens)}), flush=True)
+        return
     if args.prompt_lens:
         lo, hi = (int(v) for v in args.prompt_lens.split(":"))
         rng = random.Random(batch)

@@ -106,7 +106,7 @@ class ModelPlan:
     tie_embeddings: bool = False
     max_positions: int = 2048
     embedding_name: str = "tok_embeddings.weight"
-    final_norm_name: str = "norm.weight"
+    final_norm_name: str = "norm"               # prefix of the final norm's tensors ("norm.weight")
     head_name: str = "output.weight"
     stop_tokens: Tuple[int, ...] = ()
     # Optional steps around the layers; None leaves the step out (the reference has none

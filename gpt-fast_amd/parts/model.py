@@ -36,8 +36,9 @@ class DecoderModel:
     # ------------------------------------------------------------------ parameters
     def parameters(self) -> Dict[str, Param]:
         p = {self.plan.embedding_name: Param((self.plan.vocab_size, self.plan.dim)),
-             self.plan.head_name: Param((self.plan.vocab_size, self.plan.dim)),
-             self.plan.final_norm_name: Param((self.plan.dim,), "vector", "norm")}
+             self.plan.head_name: Param((self.plan.vocab_size, self.plan.dim))}
+        for name, param in self.final_norm.parameters().items():
+            p[f"{self.plan.final_norm_name}.{name}"] = param
         if self.input_position is not None:
             for name, param in self.input_position.parameters().items():
                 p[f"{self.plan.input_position_name}.{name}"] = param
@@ -55,7 +56,8 @@ class DecoderModel:
         self._tensors = dict(tensors)
         self.embedding = tensors[self.plan.embedding_name]
         self.head = tensors[self.plan.head_name]
-        self.final_norm.bind({"weight": tensors[self.plan.final_norm_name]})
+        prefix = self.plan.final_norm_name + "."
+        self.final_norm.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
         if self.input_position is not None:
             prefix = self.plan.input_position_name + "."
             self.input_position.bind({k[len(prefix):]: v for k, v in tensors.items()

@@ -66,8 +66,10 @@ def write_random_model(folder: str, arch, config, seed: int, dtype="bfloat16", *
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f, indent=1)
     layout = arch.bindings(config)
+    # whether the head shares the embedding table is the plan's to say, under whatever key
+    # the architecture's config.json holds it
     tensors = random_checkpoint(layout, seed, dtype, std=std, norm_std=norm_std,
-                                tie=bool(cfg.get("tie_word_embeddings", False)))
+                                tie=bool(arch.plan(config).tie_embeddings))
     write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
     return folder
 

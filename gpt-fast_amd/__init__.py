@@ -19,3 +19,17 @@ from .engine.generate import GenerationResult, generate
 from .engine.cli import main
 from .sampling import SamplingParams
 from . import config, weights, parts, cache, engine, sampling, ops
+
+
+def _import_plugins():
+    """Modules named in GPT_FAST_AMD_PLUGINS (comma-separated, importable names) are imported
+    with the package, so that architectures and parts registered outside it are known to the
+    command line and to the trace replay as well."""
+    import importlib
+    import os
+    for name in filter(None, (n.strip() for n in os.environ.get("GPT_FAST_AMD_PLUGINS", "").split(","))):
+        importlib.import_module(name)
+
+
+_import_plugins()
+

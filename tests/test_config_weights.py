@@ -420,3 +420,25 @@ def test_a_library_is_rebuilt_when_its_source_changes(tmp_path, monkeypatch):
     (tmp_path / "libgfa_toy.so.stamp").write_text(b.source_hash("toy"))
     monkeypatch.setattr(b, "FLAGS", b.FLAGS + ["-DX"])
     assert not b._is_current(str(lib), "toy")                       # flags changed
+
+
+def test_plugins_named_in_the_environment_are_imported_with_the_package(tmp_path):
+    """An architecture registered by a module outside the package is known to every program
+    of the library (command line, trace replay) when GPT_FAST_AMD_PLUGINS names the module."""
+    import subprocess
+    import sys
+    (tmp_path / "my_plugin.py").write_text(
+        "from gpt_fast_amd.config.registry import Architecture, register_architecture\n"
+        "register_architecture(Architecture(names=('PluggedIn',), read_config=dict, plan=None,\n"
+        "                                   bindings=None, config_dict=dict))\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, GPT_FAST_AMD_PLUGINS="my_plugin",
+               PYTHONPATH=os.pathsep.join([str(tmp_path), root, os.environ.get("PYTHONPATH", "")]))
+    out = subprocess.run([sys.executable, "-c",
+                          "import gpt_fast_amd as g; print('PluggedIn' in g.known_architectures())"],
+                         env=env, capture_output=True, text=True, cwd=root)
+    assert out.returncode == 0 and out.stdout.strip() == "True", out.stderr[-500:]
+    env["GPT_FAST_AMD_PLUGINS"] = "no_such_module_anywhere"
+    out = subprocess.run([sys.executable, "-c", "import gpt_fast_amd"], env=env,
+                         capture_output=True, text=True, cwd=root)
+    assert out.returncode != 0 and "no_such_module_anywhere" in out.stderr

@@ -239,3 +239,36 @@ def test_a_toy_architecture_from_its_own_config_json_to_tokens(dtype, tmp_path):
     with pytest.raises(WeightsError) as e:
         gfa.Engine.from_folder(bad, dtype=dtype, device=DEV, max_tokens=256)
     assert e.value.missing == ["stack.2.down"] and e.value.unexpected == ["stack.9.down"]
+
+
+def test_the_toy_architecture_through_the_replay_program(tmp_path):
+    """bin/trace_run knows the architecture through a plugin module named in the environment:
+    a prompt, then single tokens, from the toy folder, against the plain computation."""
+    import subprocess
+    import numpy as np
+    gfa = _register()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = str(tmp_path / "toy")
+    arch = gfa.architecture("toy_stack")
+    cfg = arch.read_config(TOY)
+    gfa.write_random_model(folder, arch, cfg, seed=6, dtype="bfloat16", std=0.08)
+    t = {k: v.float() for k, v in plain.read_safetensors(os.path.join(folder, "model.safetensors")).items()}
+    (tmp_path / "toy_plugin.py").write_text("import test_toy_architecture_gpu as T\nT._register()\n")
+    toks = util.random_tokens(cfg.vocab, 45, 8)
+    steps = [{"step": 0, "entries": [{"id": "r", "tokens": toks[:30], "want": list(range(30))}], "end": []}]
+    steps += [{"step": i - 29, "entries": [{"id": "r", "tokens": [toks[i]], "want": [0]}],
+               "end": ["r"] if i == 44 else []} for i in range(30, 45)]
+    env = dict(os.environ, GPT_FAST_AMD_PLUGINS="toy_plugin",
+               PYTHONPATH=os.pathsep.join([str(tmp_path), os.path.join(root, "tests"), root,
+                                           os.environ.get("PYTHONPATH", "")]))
+    want = _plain_logits(t, cfg, toks)
+    for dtype, tol in (("float32", TOL_F32), ("bfloat16", TOL_BF16)):
+        out = str(tmp_path / dtype)
+        proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                               "--out", out, "--max-tokens", "64"],
+                              input="\n".join(json.dumps(s) for s in steps) + "\n",
+                              capture_output=True, text=True, timeout=110, env=env)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        got = torch.cat([torch.from_numpy(np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4")
+                                          .reshape(-1, cfg.vocab).copy()) for s in steps])
+        assert rel_err(got, want) < tol, dtype

@@ -524,7 +524,8 @@ def test_dispatch_thresholds_follow_the_number_of_compute_units():
     assert A.plan(1, 1, 32, 8, 128, 3, units=256)[3] == 1          # a short context: no split
     L._units["fake256"], L._units["fake64"] = 256, 64
     try:
-        assert L._library_slices(512, 4096, 14336, "fake256") == 8
+        assert L._library_slices(512, 4096, 14336, "fake256") == 4
+        assert L._library_slices(200, 4096, 14336, "fake256") == 8
         assert L._library_slices(2048, 4096, 14336, "fake256") == 2
         assert L._library_slices(2048, 4096, 4096, "fake256") == 1
         assert L._library_slices(2048, 4096, 14336, "fake64") == 1

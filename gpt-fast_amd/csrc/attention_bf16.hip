@@ -59,16 +59,42 @@ __device__ __forceinline__ float sum_over_lane_groups(float v) {
 // position and the first 63 entries of its page row - one per lane, handed out by readlane
 // as the blocks come - are requested together, and the keys and values follow in the second
 // round.  Otherwise q_start -> position -> page number -> keys is a chain of four.
-template <int DS, int RT, bool PREFETCH, bool SINGLE = false>
+// SLICED (with SINGLE): the step's q, k and v rows are not there yet - only the float partial
+// sums [S, sequences, (H + 2 Hkv) * hd] of the sliced product that makes them.  The workgroup
+// adds the slices of its own sequence and kv head (the group's query heads, the new key, the
+// new value), rotates queries and key by the token's position (interleaved pairs, the
+// arithmetic of rope_cache_sliced_bf16x8_kernel in core.hip) and keeps them in LDS: the
+// queries become its operand, the key and value are put into the operands of the block that
+// holds the token's position after that block's loads, and the workgroup of the last split
+// writes them to the cache for the steps to come.  The rotation and cache-write kernel and
+// its round trip through memory fall away.
+struct SlicedRowsIn {
+    const float* part;        // null unless SLICED
+    int S;
+    size_t slice;             // elements between slices
+    int width;                // (H + 2 Hkv) * hd
+    const float* freqs;       // [rot / 2], null if rot == 0
+    int rot;
+    bf16_t* k_out;            // the caches again, to write to
+    bf16_t* v_out;
+};
+#define SL_MAX_ROT 256
+#define SL_MAX_ELEMS (18 * 128)           // sixteen query heads, key, value of up to 128 dims
+
+template <int DS, int RT, bool PREFETCH, bool SINGLE = false, bool SLICED = false>
 __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table, int table_stride,
         bf16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml, int H,
-        int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows, int out_pad) {
+        int Hkv, int hd, float scale_log2, int window, int n_splits, int total_rows, int out_pad,
+        SlicedRowsIn sl) {
     constexpr int DT = DS * 2;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     static_assert(!SINGLE || RT == 1, "one token per sequence is one tile of rows");
+    static_assert(!SLICED || SINGLE, "partial sums are taken for one token per sequence");
+    __shared__ float sl_cs[SLICED ? SL_MAX_ROT : 1];                             // cos, sin per pair
+    __shared__ __attribute__((aligned(16))) bf16_t sl_rows[SLICED ? SL_MAX_ELEMS : 8];   // q heads, k, v
     const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
     // SINGLE: lane i < 63 holds entry i of the page row and lane 63 the sequence's position,
     // from one load instruction that needs only arguments which arrive in registers; it is
@@ -102,6 +128,58 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
     const int* pages = table + (size_t)seq * table_stride;
     const int spos = SINGLE ? __builtin_amdgcn_readlane(first_pages, 63) : start_pos[seq];
 
+    if (SLICED) {
+        // four elements at a time: R query heads of this group, then the key, then the value.
+        // A thread's first four are requested before the table of cosines and sines is made
+        // (their addresses need no position), so the two round trips overlap.
+        const int per_head = hd >> 2, n_items = (R + 2) * per_head;
+        const float* row = sl.part + (size_t)seq * sl.width;
+        auto column = [&](int i) {
+            const int head = i / per_head, d = (i - head * per_head) * 4;
+            return (head < R ? g * R + head : head == R ? H + g : H + Hkv + g) * hd + d;
+        };
+        auto summed = [&](int i) {
+            const int col = column(i);
+            float4 a = *(const float4*)(row + col);
+            for (int sidx = 1; sidx < sl.S; ++sidx) {
+                const float4 b = *(const float4*)(row + (size_t)sidx * sl.slice + col);
+                a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+            }
+            return a;
+        };
+        auto rotate_and_keep = [&](int i, float4 a) {
+            const int head = i / per_head, d = (i - head * per_head) * 4;
+            if (head <= R && d < sl.rot) {
+                const float c0 = sl_cs[d], s0 = sl_cs[d + 1], c1 = sl_cs[d + 2], s1 = sl_cs[d + 3];
+                a = make_float4(a.x * c0 - a.y * s0, a.y * c0 + a.x * s0,
+                                a.z * c1 - a.w * s1, a.w * c1 + a.z * s1);
+            }
+            union { uint2 u; bf16_t e[4]; } w;
+            w.e[0] = float_to_bf16(a.x); w.e[1] = float_to_bf16(a.y);
+            w.e[2] = float_to_bf16(a.z); w.e[3] = float_to_bf16(a.w);
+            *(uint2*)(sl_rows + head * hd + d) = w.u;
+        };
+        const int first = threadIdx.x;
+        float4 a_first = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (first < n_items) a_first = summed(first);
+        for (int i = threadIdx.x; i < sl.rot / 2; i += blockDim.x)
+            sincosf((float)spos * sl.freqs[i], &sl_cs[2 * i + 1], &sl_cs[2 * i]);
+        __syncthreads();
+        if (first < n_items) rotate_and_keep(first, a_first);
+        for (int i = first + blockDim.x; i < n_items; i += blockDim.x) rotate_and_keep(i, summed(i));
+        __syncthreads();
+        if (split == n_splits - 1 && wave == 0 && sl.k_out) {
+            // the new key and value go to their place in the cache (the reads of this step
+            // take them from LDS: this write need not have landed)
+            const int pi = spos >> 6, off = spos & (GFA_PAGE - 1);
+            const int page = pi < 63 ? __builtin_amdgcn_readlane(first_pages, pi < 63 ? pi : 0) : pages[pi];
+            if (lane < (hd >> 3))
+                *(uint4*)(sl.k_out + key_elem(page, g, off, lane * 8, Hkv, hd)) = *(const uint4*)(sl_rows + R * hd + lane * 8);
+            for (int d = lane; d < hd; d += 64)
+                sl.v_out[value_elem(page, g, d, off, Hkv, hd)] = sl_rows[(R + 1) * hd + d];
+        }
+    }
+
     Frag qf[RT][DS];
     int rpos[RT];             // position of this lane's row in tile rt, -1 if there is none
     size_t orow[RT];          // (token, head) index of that row in q / out
@@ -112,7 +190,7 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
         const int t = (valid && !SINGLE) ? r / R : 0, hh = valid ? r - t * R : 0;
         rpos[rt] = valid ? spos + t : -1;
         orow[rt] = (size_t)(q0 + t) * H + g * R + hh;
-        const bf16_t* qrow = q + orow[rt] * hd;
+        const bf16_t* qrow = SLICED ? sl_rows + hh * hd : q + orow[rt] * hd;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const int d = ds * 32 + lg * 8;
@@ -168,6 +246,30 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
     };
     auto compute_block = [&](int kb, Frag (&kf)[2][DS], Frag (&vf)[DT]) {
         const int key0 = kb * 32 + lg * 8;                 // this lane's keys: key0 .. key0 + 7
+        if (SLICED && kb == (pmax >> 5)) {
+            // the block of the token itself: its key and value come from LDS, whatever the
+            // cache held at their place when the block was loaded
+            const int in_block = pmax & 31, slot = key_slot(in_block);
+            if (li == (slot & 15)) {
+#pragma unroll
+                for (int ds = 0; ds < DS; ++ds) {
+                    const int d = ds * 32 + lg * 8;
+                    if (d < hd) {
+                        const uint4 knew = *(const uint4*)(sl_rows + R * hd + d);
+                        if (slot >> 4) kf[1][ds].u = knew; else kf[0][ds].u = knew;
+                    }
+                }
+            }
+            if (lg == (in_block >> 3)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const bf16_t vnew = sl_rows[(R + 1) * hd + (dt * 16 < hd ? dt * 16 : 0) + li];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (e == (in_block & 7)) vf[dt].e[e] = vnew;
+                }
+            }
+        }
         floatx4_t s[RT][2];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
@@ -838,13 +940,13 @@ static void launch_attention(int rt, int nw, dim3 grid, hipStream_t stream, cons
                              int n_splits, int total_rows, bool single, int out_pad) {
     const size_t shmem = nw > 1 ? (size_t)(nw - 1) * rt * (16 * 2 * sizeof(float) + DS * 2 * 64 * sizeof(floatx4_t)) : 0;
     if (rt == 1 && single)
-        attention_mfma_kernel<DS, 1, false, true><<<dim3(n_splits, grid.y, grid.z / n_splits), 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, out_pad);
+        attention_mfma_kernel<DS, 1, false, true><<<dim3(n_splits, grid.y, grid.z / n_splits), 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, out_pad, SlicedRowsIn{});
     else if (rt == 1)
-        attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
+        attention_mfma_kernel<DS, 1, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0, SlicedRowsIn{});
     else if (rt == 2)
-        attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
+        attention_mfma_kernel<DS, 2, (DS <= 4)><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0, SlicedRowsIn{});
     else if (DS <= 4)
-        attention_mfma_kernel<(DS <= 4 ? DS : 4), 4, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0);
+        attention_mfma_kernel<(DS <= 4 ? DS : 4), 4, false><<<grid, 64 * nw, shmem, stream>>>(q, k, v, q_start, start_pos, table, table_stride, out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, 0, SlicedRowsIn{});
 }
 
 // q, out [n_tokens, H, hd]; the sequences' token runs are given by q_start [n_seqs + 1] and
@@ -889,5 +991,50 @@ extern "C" int gfa_attention_bf16(const void* q, const void* k_pages, const void
         launch_attention<8>(rt, n_waves, grid, stream, qp, kp, vp, q_start, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv, hd, sl2, window, n_splits, total_rows, single, out_pad);
     if (n_splits > 1)
         attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows, H, out_pad);
+    return GFA_LAUNCH_RESULT();
+}
+
+// One token per sequence whose q, k and v rows are still the float partial sums part
+// [S, n_seqs, (H + 2 Hkv) * hd] of a sliced product: the slices are added, queries and key
+// rotated (interleaved pairs, rot a multiple of 4, frequencies freqs [rot / 2]) and attended in
+// one kernel, and the new keys and values written to the cache (k_pages / v_pages; a run that
+// reads another run's cache gives write_cache = 0).  out [n_seqs, H, hd]; start_pos [n_seqs] is
+// each token's position; head sizes up to 128, at most sixteen query heads per kv head.
+extern "C" int gfa_attention_sliced_bf16(const float* part, int S, const float* freqs, int rot,
+                                         void* k_pages, void* v_pages, int write_cache,
+                                         const int* start_pos, const int* table, int table_stride,
+                                         void* out, float* ws_o, float* ws_ml, int n_seqs, int H,
+                                         int Hkv, int hd, float scale, int window, int n_waves,
+                                         int n_splits, hipStream_t stream) {
+    if (n_seqs <= 0) return 0;
+    if ((long)table_stride * 2 * (n_splits + 1) >= (1L << 31)) return (int)hipErrorInvalidValue;
+    if (!part || S < 1 || hd % 16 != 0 || hd > 128 || Hkv < 1 || H % Hkv != 0 || H / Hkv > 16 ||
+        rot < 0 || rot % 4 != 0 || rot > hd || rot > SL_MAX_ROT || (rot > 0 && !freqs) ||
+        (H / Hkv + 2) * hd > SL_MAX_ELEMS || n_splits < 1 || n_splits > 64 || !(scale > 0.f) ||
+        (n_splits > 1 && (!ws_o || !ws_ml)) || n_waves < 1 || n_waves > 8 ||
+        (size_t)(n_waves - 1) * (128 + (hd <= 64 ? 2 : 4) * 2 * 1024) > 65536)
+        return (int)hipErrorInvalidValue;
+    const int width = (H + 2 * Hkv) * hd;
+    const SlicedRowsIn sl = {part, S, (size_t)n_seqs * width, width, freqs, rot,
+                             write_cache ? (bf16_t*)k_pages : nullptr,
+                             write_cache ? (bf16_t*)v_pages : nullptr};
+    const float sl2 = scale * LOG2E;
+    const int total_rows = n_seqs * H;
+    const dim3 grid(n_splits, Hkv, n_seqs);
+    const bf16_t* kp = (const bf16_t*)k_pages;
+    const bf16_t* vp = (const bf16_t*)v_pages;
+    if (hd <= 64) {
+        const size_t shmem = n_waves > 1 ? (size_t)(n_waves - 1) * (16 * 2 * sizeof(float) + 2 * 2 * 64 * sizeof(floatx4_t)) : 0;
+        attention_mfma_kernel<2, 1, false, true, true><<<grid, 64 * n_waves, shmem, stream>>>(
+            nullptr, kp, vp, nullptr, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv,
+            hd, sl2, window, n_splits, total_rows, 0, sl);
+    } else {
+        const size_t shmem = n_waves > 1 ? (size_t)(n_waves - 1) * (16 * 2 * sizeof(float) + 4 * 2 * 64 * sizeof(floatx4_t)) : 0;
+        attention_mfma_kernel<4, 1, false, true, true><<<grid, 64 * n_waves, shmem, stream>>>(
+            nullptr, kp, vp, nullptr, start_pos, table, table_stride, (bf16_t*)out, ws_o, ws_ml, H, Hkv,
+            hd, sl2, window, n_splits, total_rows, 0, sl);
+    }
+    if (n_splits > 1)
+        attention_combine_kernel<<<total_rows, 64, 0, stream>>>(ws_o, ws_ml, (bf16_t*)out, hd, n_splits, total_rows, H, 0);
     return GFA_LAUNCH_RESULT();
 }

@@ -116,3 +116,40 @@ def attention(q, k_pages, v_pages, batch, table, scale, window, chunked: bool = 
         "attention_bf16")
     return res
 
+
+def attention_sliced(part, freqs, rot: int, k_pages, v_pages, write_cache: bool, batch, table,
+                     scale: float, window: int, H: int):
+    """One token per sequence whose q, k and v rows are still the float32 partial sums ``part``
+    [S, N, (H + 2 G) * hd] of a sliced product: the slices are added, queries and keys rotated
+    (interleaved pairs; ``freqs`` [rot / 2]), the new keys and values written to the cache
+    (unless ``write_cache`` is false) and attended, in one kernel.  Returns [N, H, hd]
+    bfloat16, or None if the kernel does not take this step (the caller then rotates and
+    attends with the kernels of their own)."""
+    S, n, width = part.shape
+    G = k_pages.shape[1]
+    hd = width // (H + 2 * G) if H + 2 * G else 0
+    if (batch.max_q_len != 1 or n != batch.n_seqs or hd % 16 or hd > 128 or H % G or H // G > 16
+            or rot % 4 or rot > hd or width != (H + 2 * G) * hd or part.dtype != torch.float32
+            or k_pages.dtype != torch.bfloat16 or table.shape[1] * 2 * 65 >= 1 << 31):
+        return None
+    require_device(part, k_pages, v_pages, table, batch.start_pos, *([freqs] if rot else []))
+    require_contiguous(part=part, k_pages=k_pages, v_pages=v_pages, table=table)
+    if tuple(k_pages.shape[1:]) != (G, 64, hd) or tuple(v_pages.shape[1:]) != (G, hd, 64):
+        raise KernelError(f"attention_sliced: pages are {tuple(k_pages.shape)} / {tuple(v_pages.shape)}")
+    if rot and (freqs.dtype != torch.float32 or freqs.numel() != rot // 2 or not freqs.is_contiguous()):
+        raise KernelError("attention_sliced: one float32 frequency per rotated pair")
+    if batch.start_pos.numel() != n or table.shape[0] < n or table.dtype != torch.int32:
+        raise KernelError("attention_sliced: one position and one table row per sequence")
+    rt, nw, tiles, splits = plan(n, 1, H, G, hd, table.shape[1])
+    out = torch.empty((n, H, hd), dtype=torch.bfloat16, device=part.device)
+    ws_o = ws_ml = None
+    if splits > 1:
+        ws_o = torch.empty((splits, n * H, hd), dtype=torch.float32, device=part.device)
+        ws_ml = torch.empty((splits, n * H, 2), dtype=torch.float32, device=part.device)
+    check(library("attention_bf16").gfa_attention_sliced_bf16(
+        ptr(part), _i(S), ptr(freqs) if rot else None, _i(rot), ptr(k_pages), ptr(v_pages),
+        _i(int(bool(write_cache))), ptr(batch.start_pos), ptr(table), _i(table.shape[1]), ptr(out),
+        ptr(ws_o), ptr(ws_ml), _i(n), _i(H), _i(G), _i(hd), _f(scale), _i(window), _i(nw), _i(splits),
+        stream_handle()), "attention_sliced_bf16")
+    return out
+

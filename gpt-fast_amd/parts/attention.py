@@ -75,6 +75,17 @@ class Attention(Part):
         if q is None:
             qkv = L.linear(x, self.wqkv,                                    # model.py:195
                            may_stay_sliced=getattr(self.position, "takes_sliced", False))
+            whole = getattr(self.position, "rotate_store_attend", None)
+            if whole is not None and isinstance(qkv, L.SlicedRows):
+                # one token per sequence, the projection still in slices: rotation, cache
+                # write and attention as one kernel (model.py:201-211)
+                y = whole(qkv, batch, entry, s.n_heads, s.n_kv_heads, s.head_dim, self.scale,
+                          self.window)
+                if y is not None:
+                    y = y.view(n_rows, s.n_heads * s.head_dim)
+                    add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
+                        y, self.wo, rows, then_norm, takes_halves))           # model.py:215, 162
+                    return
             q = self.position.rotate_and_store(qkv, batch, entry, s.n_heads, s.n_kv_heads,
                                                s.head_dim)                  # model.py:201-207
 

@@ -81,6 +81,20 @@ class RotaryPosition(Part):
             qkv, self.freqs, batch.tok_seq, batch.tok_pos, batch.table(entry.group_id), *pages,
             n_heads, n_kv_heads, head_dim, self.spec.rotary_dim, self.LAYOUTS[self.spec.layout])
 
+    def rotate_store_attend(self, qkv, batch, entry, n_heads, n_kv_heads, head_dim, scale, window):
+        """For a step of one token per sequence whose ``qkv`` is still an
+        ``ops.linear.SlicedRows``: rotation, cache write and attention in one kernel.  None:
+        not available for this step (the caller rotates, stores and attends apart)."""
+        # a run that reads another run's cache attends to that run's keys and values, also at
+        # the token's own position: not to the ones this kernel would make of its own rows
+        if (self.spec.layout != "interleaved" or not isinstance(qkv, L.SlicedRows)
+                or qkv.dtype != torch.bfloat16 or entry is None or not entry.writes):
+            return None
+        from ..ops import attention_bf16 as AB
+        return AB.attention_sliced(qkv.part, self.freqs, self.spec.rotary_dim, entry.k_pages,
+                                   entry.v_pages, True, batch, batch.table(entry.group_id),
+                                   scale, window or 0, n_heads)
+
     def project_rotate_store(self, x, wqkv, batch, entry, n_heads, n_kv_heads, head_dim):
         """Projection + rotation + cache write in one kernel for few rows (interleaved
         pairs only: both elements of a pair are then in one lane).  None: not available."""

@@ -734,6 +734,64 @@ def test_rope_and_cache_write_over_partial_sums(H, G, hd, rot, S):
         close(vc[page, :, :, p % 64], ref[n, H + G:], 1e-2)
 
 
+@pytest.mark.parametrize("H,G,hd,rot,S", [(32, 8, 128, 128, 4), (6, 2, 32, 16, 3), (4, 4, 64, 64, 1),
+                                          (16, 1, 16, 0, 2), (12, 3, 48, 24, 2)])
+def test_attention_over_partial_sums_of_the_projection(H, G, hd, rot, S):
+    """One token per sequence, q, k and v still as the float partial sums of a sliced product:
+    one kernel adds the slices, rotates, writes the new key and value to the cache and attends.
+    Against float64 of the whole: the summed rows, rotated by interleaved pairs, the token's
+    own key and value among the sequence's (contexts that end at a block's and a page's first
+    and last places, long enough for context splits; dirty places behind the newest key)."""
+    from gpt_fast_amd.ops import attention_bf16 as A
+    torch.manual_seed(H + hd)
+    ctx = [1, 32, 33, 64, 65, 200, 1000, 2049][:8]          # keys including the new one
+    n = len(ctx)
+    k_pages, v_pages, table, ks, vs = _paged(ctx, G, hd, torch.bfloat16, 5)
+    part = torch.randn(S, n, (H + 2 * G) * hd)
+    freqs = 1.0 / (10000.0 ** (torch.arange(0, rot, 2).float() / max(rot, 1)))
+    rows = part.double().sum(0).view(n, H + 2 * G, hd)
+    pos = torch.tensor([c - 1 for c in ctx], dtype=torch.float32)
+    ref = rows.clone()
+    if rot:
+        ang = pos[:, None] * freqs[None, :]
+        c, s_ = torch.cos(ang.double())[:, None, :], torch.sin(ang.double())[:, None, :]
+        a, b = rows[:, :H + G, 0:rot:2], rows[:, :H + G, 1:rot:2]
+        ref[:, :H + G, 0:rot:2] = a * c - b * s_
+        ref[:, :H + G, 1:rot:2] = b * c + a * s_
+    q, k_new, v_new = ref[:, :H], ref[:, H:H + G], ref[:, H + G:]
+
+    class Step:
+        n_seqs, max_q_len = n, 1
+        start_pos = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+
+    kp, vp = k_pages.clone(), v_pages.clone()
+    out = A.attention_sliced(part.to(DEV), freqs.to(DEV) if rot else None, rot, kp, vp, True, Step,
+                             table, 1.0 / math.sqrt(hd), 0, H)
+    table, k_pages, v_pages = table.cpu(), k_pages.cpu(), v_pages.cpu()
+    assert out is not None and out.shape == (n, H, hd)
+    kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
+    R = H // G
+    for b_ in range(n):
+        # the sequence's earlier keys and values as the cache holds them, the new ones as computed
+        K_ = torch.cat([ks[b_][:ctx[b_] - 1].double(), k_new[b_][None]], 0)        # [ctx, G, hd]
+        V_ = torch.cat([vs[b_][:ctx[b_] - 1].double(), v_new[b_][None]], 0)
+        for h in range(H):
+            g = h // R
+            sc = (K_[:, g] @ q[b_, h]) / math.sqrt(hd)
+            want = torch.softmax(sc, 0) @ V_[:, g]
+            close(out[b_, h], want, 2e-2)
+        page = int(table[b_, (ctx[b_] - 1) // 64])
+        close(kc[page, :, (ctx[b_] - 1) % 64], k_new[b_], 1e-2)                  # written for later steps
+        close(vc[page, :, :, (ctx[b_] - 1) % 64], v_new[b_], 1e-2)
+    # nothing else in the cache changed
+    k0, v0 = from_cache_order(k_pages.float(), v_pages.float())
+    for b_ in range(n):
+        page, off = int(table[b_, (ctx[b_] - 1) // 64]), (ctx[b_] - 1) % 64
+        k0[page, :, off], v0[page, :, :, off] = kc[page, :, off], vc[page, :, :, off]
+    assert torch.equal(torch.nan_to_num(k0, nan=7.0), torch.nan_to_num(kc, nan=7.0))
+    assert torch.equal(torch.nan_to_num(v0, nan=7.0), torch.nan_to_num(vc, nan=7.0))
+
+
 def test_argmax_and_sampling():
     from gpt_fast_amd.sampling import SamplingParams, logits_to_probs, sample
     import plain_llama as plain

@@ -734,9 +734,10 @@ def test_rope_and_cache_write_over_partial_sums(H, G, hd, rot, S):
         close(vc[page, :, :, p % 64], ref[n, H + G:], 1e-2)
 
 
+@pytest.mark.parametrize("window", [0, 50])
 @pytest.mark.parametrize("H,G,hd,rot,S", [(32, 8, 128, 128, 4), (6, 2, 32, 16, 3), (4, 4, 64, 64, 1),
                                           (16, 1, 16, 0, 2), (12, 3, 48, 24, 2)])
-def test_attention_over_partial_sums_of_the_projection(H, G, hd, rot, S):
+def test_attention_over_partial_sums_of_the_projection(H, G, hd, rot, S, window):
     """One token per sequence, q, k and v still as the float partial sums of a sliced product:
     one kernel adds the slices, rotates, writes the new key and value to the cache and attends.
     Against float64 of the whole: the summed rows, rotated by interleaved pairs, the token's
@@ -766,7 +767,7 @@ def test_attention_over_partial_sums_of_the_projection(H, G, hd, rot, S):
 
     kp, vp = k_pages.clone(), v_pages.clone()
     out = A.attention_sliced(part.to(DEV), freqs.to(DEV) if rot else None, rot, kp, vp, True, Step,
-                             table, 1.0 / math.sqrt(hd), 0, H)
+                             table, 1.0 / math.sqrt(hd), window, H)
     table, k_pages, v_pages = table.cpu(), k_pages.cpu(), v_pages.cpu()
     assert out is not None and out.shape == (n, H, hd)
     kc, vc = from_cache_order(kp.cpu().float(), vp.cpu().float())
@@ -775,10 +776,11 @@ def test_attention_over_partial_sums_of_the_projection(H, G, hd, rot, S):
         # the sequence's earlier keys and values as the cache holds them, the new ones as computed
         K_ = torch.cat([ks[b_][:ctx[b_] - 1].double(), k_new[b_][None]], 0)        # [ctx, G, hd]
         V_ = torch.cat([vs[b_][:ctx[b_] - 1].double(), v_new[b_][None]], 0)
+        first = max(0, ctx[b_] - window) if window else 0     # keys at distance < window
         for h in range(H):
             g = h // R
-            sc = (K_[:, g] @ q[b_, h]) / math.sqrt(hd)
-            want = torch.softmax(sc, 0) @ V_[:, g]
+            sc = (K_[first:, g] @ q[b_, h]) / math.sqrt(hd)
+            want = torch.softmax(sc, 0) @ V_[first:, g]
             close(out[b_, h], want, 2e-2)
         page = int(table[b_, (ctx[b_] - 1) // 64])
         close(kc[page, :, (ctx[b_] - 1) % 64], k_new[b_], 1e-2)                  # written for later steps

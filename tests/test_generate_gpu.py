@@ -689,3 +689,47 @@ def test_command_line_interactive_streams_the_answer(tmp_path_factory, tmp_path)
         inv = {i: t for t, i in vocab.items()}
         assert "".join(" " + inv[t] for t in want) in proc.stdout, proc.stdout[-800:]
         assert f"Prompt Length: 3" in proc.stdout          # of the warm-up prompt, BOS included
+
+
+def test_windowed_layers_at_twenty_rows(tmp_path_factory):
+    """The same three kinds of layer with twenty sequences decoding at once: a step of twenty
+    rows runs on the tiled-weight products and the attention kernel that adds the projection's
+    slices itself, with windows, while windowed groups give pages back (their table entries
+    turn -1).  bfloat16 against the plain model with the same windows."""
+    import dataclasses
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd import Entry
+    from gpt_fast_amd.weights.bindings import load_parameters
+    folder = util.make_folder(tmp_path_factory.getbasetemp(), "B", dtype="bfloat16")
+    arch, cfg = gfa.read_model_folder(folder)
+    plan = arch.plan(cfg)
+    windows = [None, 70, 20]
+    plan.layers = [dataclasses.replace(layer, mixer=dataclasses.replace(layer.mixer, window=win))
+                   for layer, win in zip(plan.layers, windows)]
+    params = load_parameters(folder, arch.bindings(cfg), "bfloat16", torch.device("cuda:0"))
+    eng = gfa.Engine.from_plan(plan, params, "bfloat16", "cuda:0", max_tokens=64 * 20 * 4,
+                               max_sequences=20)
+    pcfg, w = plain.load_folder(folder)
+    n_seq, new = 20, 40
+    prompts = [60 + 7 * i for i in range(n_seq)]                       # 60 .. 193 tokens
+    seqs = [util.random_tokens(pcfg["vocab"], prompts[i] + new, 40 + i) for i in range(n_seq)]
+    slots = [eng.start_sequence() for _ in range(n_seq)]
+    got = [[] for _ in range(n_seq)]
+    for lo in range(0, n_seq, 5):                                      # prompts five at a time
+        out = eng.step([Entry(slots[i], seqs[i][:prompts[i]], want=[prompts[i] - 1])
+                        for i in range(lo, lo + 5)]).cpu()
+        for j, i in enumerate(range(lo, lo + 5)):
+            got[i].append(out[j])
+    for t in range(new - 1):
+        out = eng.step([Entry(slots[i], [seqs[i][prompts[i] + t]], want=[0]) for i in range(n_seq)]).cpu()
+        for i in range(n_seq):
+            got[i].append(out[i])
+    for i in (0, 7, 13, 19):
+        want = _plain_forward_with_windows(w, pcfg, seqs[i][:-1], windows)[prompts[i] - 1:]
+        assert rel_err(torch.stack(got[i]), want) < TOL_BF16, i
+    gone = [sum(1 for p in eng.cache.page_list(gid, slots[19]) if p < 0)
+            for gid, g in eng.cache.kv_groups if g.need.window == 20]
+    assert gone and gone[0] >= 2                                        # pages did go back
+    eng.cache.check()
+    for s in slots:
+        eng.end_sequence(s)
